@@ -1,0 +1,302 @@
+"""CPU oracle for the FP8/FP4 quantisation path (TEST INFRASTRUCTURE, not product code).
+
+This module restates, with plain PyTorch CPU ops, the arithmetic of the reference's
+pure-torch implementations:
+
+* ``cast`` / ``cast_back``      <- tile_kernels/torch/cast.py:62-221 and :40-59
+* ``swiglu_forward``            <- tile_kernels/torch/swiglu.py:9-88
+* ``unpack_from_e2m1fn_x2``     <- tile_kernels/quant/common.py:247-295
+* ``encode_e2m1``               <- tile_kernels/torch/cast.py:224-252 (same result, closed form)
+
+Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import
+it.  The shipped package never does: it has no CPU path at all.
+
+How each function is pinned (all pins live in tests/test_oracle_*.py and run without a GPU):
+
+* E4M3 encoding goes through ``Tensor.to(torch.float8_e4m3fn)``; it is checked against an
+  independent nearest-ties-to-even search over the 256-entry OCP E4M3FN value table for every
+  bf16 bit pattern and for fp32 midpoints/neighbours, plus hand known answers.
+* ``encode_e2m1`` is a threshold formula; it is checked against a brute-force nearest/ties-to-
+  even-code search over the 16-entry E2M1 table and against hand known answers.
+* scale arithmetic is checked against closed forms (amax 448 -> 1.0, zero group -> clamp/448,
+  the integer identity for power-of-two rounding over every exponent).
+* block geometry / partial blocks / scale layouts are checked against a naive Python double
+  loop on tiny inputs and against stride/shape invariants.
+* the whole of ``cast`` is cross-checked bit-for-bit against the independent scalar C
+  restatement in oracle/quant_ref.c.
+* ``swiglu_forward`` is checked against float64 evaluation and ``torch.nn.functional.silu``.
+"""
+from typing import Optional, Tuple, Union
+
+import torch
+
+QuantTensor = Tuple[torch.Tensor, torch.Tensor]
+
+E4M3_MAX = 448.0
+E2M1_MAX = 6.0
+E4M3_AMAX_FLOOR = 1e-4
+E2M1_AMAX_FLOOR = 6.0 * 2.0 ** -126
+
+# magnitudes of the eight E2M1 codes, index = 3-bit code (exp:2 | mant:1)
+E2M1_VALUES = (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0)
+
+
+def _ceil_div(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+def _round_up(a: int, b: int) -> int:
+    return _ceil_div(a, b) * b
+
+
+def _fmt_constants(fmt: str):
+    if fmt == 'e4m3':
+        return torch.float8_e4m3fn, E4M3_MAX, E4M3_AMAX_FLOOR
+    if fmt == 'e2m1':
+        return torch.int8, E2M1_MAX, E2M1_AMAX_FLOOR
+    raise AssertionError(f'unsupported format {fmt}')
+
+
+def unpack_from_e2m1fn_x2(x: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """Decode bytes holding two E2M1 codes (even element in the low nibble) to floats.
+
+    Follows tile_kernels/quant/common.py:247-295: code = s(1) e(2) m(1), bias 1.
+    """
+    assert x.dtype in (torch.int8, torch.uint8) and x.ndim >= 1
+    table = torch.tensor(E2M1_VALUES + tuple(-v for v in E2M1_VALUES), dtype=torch.float32, device=x.device)
+    b = x.view(torch.uint8).to(torch.int64)
+    pair = torch.stack((table[b & 0xF], table[(b >> 4) & 0xF]), dim=-1)
+    return pair.reshape(*x.shape[:-1], x.shape[-1] * 2).to(out_dtype)
+
+
+def encode_e2m1(q: torch.Tensor) -> torch.Tensor:
+    """fp32 -> 4-bit E2M1 code (uint8, sign in bit 3), round-to-nearest, ties to the even code,
+    saturating at 6.  Same mapping as tile_kernels/torch/cast.py:224-252.
+
+    The seven decision points between neighbouring magnitudes are .25 .75 1.25 1.75 2.5 3.5 5;
+    a tie moves up exactly when the upper neighbour has an even code (.75 1.75 3.5).
+    """
+    assert q.dtype == torch.float32
+    a = q.abs()
+    code = ((a > 0.25).to(torch.uint8) + (a >= 0.75).to(torch.uint8) + (a > 1.25).to(torch.uint8)
+            + (a >= 1.75).to(torch.uint8) + (a > 2.5).to(torch.uint8) + (a >= 3.5).to(torch.uint8)
+            + (a > 5.0).to(torch.uint8))
+    code = torch.where(torch.isnan(q), torch.full_like(code, 7), code)  # exponent 255 saturates (cast.py:247-249)
+    return code | (torch.signbit(q).to(torch.uint8) << 3)
+
+
+def _sf_as_fp32(sf: torch.Tensor) -> torch.Tensor:
+    """Scale tensor in any of the three layouts -> dense row-major fp32 (cast.py:27-37)."""
+    if sf.dtype == torch.float32:
+        return sf
+    assert sf.dtype == torch.int32
+    rows, words = sf.shape
+    # a [rows, 1] view with strides (1, ld) passes for contiguous, so copy into fresh storage instead
+    dense = torch.empty((rows, words), dtype=torch.int32).copy_(sf).view(torch.uint8).reshape(rows, words * 4)
+    return (dense.to(torch.int32) << 23).view(torch.float32)
+
+
+def _dequantise(x: QuantTensor, blk: Tuple[int, int]) -> torch.Tensor:
+    codes, sf = x
+    assert codes.dtype in (torch.float8_e4m3fn, torch.int8)
+    vals = unpack_from_e2m1fn_x2(codes) if codes.dtype == torch.int8 else codes.to(torch.float32)
+    scale = _sf_as_fp32(sf).repeat_interleave(blk[0], 0).repeat_interleave(blk[1], 1)
+    return vals * scale[: vals.shape[0], : vals.shape[1]]
+
+
+def cast_back(x: QuantTensor, fmt: str, block_size: Tuple[int, int] = (32, 32)) -> torch.Tensor:
+    """Dequantise ``(codes, scales)`` to fp32 or bf16 (tile_kernels/torch/cast.py:40-59)."""
+    out = _dequantise(x, block_size)
+    return out.to(torch.float32 if fmt == 'fp32' else torch.bfloat16)
+
+
+def _block_amax(xf: torch.Tensor, bh: int, bw: int) -> torch.Tensor:
+    """max |x| over every (bh x bw) block, partial edge blocks over their in-range part only."""
+    h, w = xf.shape
+    nm, nk = _ceil_div(h, bh), _ceil_div(w, bw)
+    canvas = xf.new_zeros((nm * bh, nk * bw))   # |x| >= 0, so zero fill never wins a max it should lose
+    canvas[:h, :w] = xf.abs()
+    return canvas.view(nm, bh, nk, bw).amax(dim=(1, 3))
+
+
+def _expand_blocks(t: torch.Tensor, bh: int, bw: int, h: int, w: int) -> torch.Tensor:
+    return t.repeat_interleave(bh, 0).repeat_interleave(bw, 1)[:h, :w]
+
+
+def _format_sf(sf_bits: torch.Tensor, col_major: bool, packed: bool) -> torch.Tensor:
+    """int32 bit patterns of the per-block dequant scales [nm, nk] -> returned scale tensor.
+
+    Layouts (tile_kernels/torch/cast.py:201-219, tile_kernels/quant/common.py:130-193):
+      row-major : fp32 [nm, nk] contiguous
+      col-major : fp32 [nm, nk], strides (1, round_up(nm, 4))
+      packed    : int32 [nm, ceil(nk/4)], strides (1, round_up(nm, 4)); byte t of word [m, j] is the
+                  biased exponent of group 4j+t, zero beyond nk
+    """
+    nm, nk = sf_bits.shape
+    if not col_major:
+        return sf_bits.view(torch.float32)
+    ld = _round_up(nm, 4)
+    if packed:
+        nw = _ceil_div(nk, 4)
+        expo = torch.zeros((ld, nw * 4), dtype=torch.uint8)
+        expo[:nm, :nk] = (sf_bits >> 23).to(torch.uint8)
+        words = expo.view(torch.int32)                       # [ld, nw], little endian byte t = group 4j+t
+        store = torch.zeros((nw, ld), dtype=torch.int32)
+        store.copy_(words.T)
+        return store.T[:nm]
+    store = torch.zeros((nk, ld), dtype=torch.float32)
+    store[:, :nm] = sf_bits.view(torch.float32).T
+    return store.T[:nm]
+
+
+def cast(
+    x: Union[torch.Tensor, QuantTensor],
+    fmt: str,
+    block_size: Tuple[int, int] = (32, 32),
+    sf: Optional[torch.Tensor] = None,
+    x_block_size: Optional[Tuple[int, int]] = None,
+    round_sf: bool = False,
+    use_tma_aligned_col_major_sf: bool = False,
+    use_packed_ue8m0: bool = False,
+    amax_floor: Optional[float] = None,
+) -> Union[torch.Tensor, QuantTensor]:
+    """Quantise a 2-D tensor to E4M3 or packed E2M1 with one scale per (bh x bw) block.
+
+    Same arguments and results as the reference's ``tile_kernels.torch.cast``
+    (tile_kernels/torch/cast.py:62-221).  ``amax_floor`` additionally lets a caller override the
+    lower clamp of the block amax, which the fused SwiGLU op exposes as ``sf_clamp_min``
+    (tile_kernels/quant/swiglu_forward_and_per_token_cast_kernel.py:234-236).
+    """
+    requant = isinstance(x, tuple)
+    if requant:
+        assert x_block_size is not None
+        xf = _dequantise(x, x_block_size)
+    else:
+        assert x.dtype in (torch.bfloat16, torch.float32)
+        xf = x.to(torch.float32)
+    assert xf.ndim == 2
+    h, w = xf.shape
+    bh, bw = block_size
+    code_dtype, qmax, floor = _fmt_constants(fmt)
+    if amax_floor is not None:
+        floor = amax_floor
+    fp4 = fmt == 'e2m1'
+    nm, nk = _ceil_div(h, bh), _ceil_div(w, bw)
+
+    if h == 0:   # cast.py:110-123
+        codes = torch.empty((0, w // 2 if fp4 else w), dtype=code_dtype)
+        if sf is not None:
+            return codes
+        if use_packed_ue8m0:
+            return codes, torch.empty((_ceil_div(nk, 4), 0), dtype=torch.int32).T
+        if use_tma_aligned_col_major_sf:
+            return codes, torch.empty((nk, 0), dtype=torch.float32).T
+        return codes, torch.empty((0, nk), dtype=torch.float32)
+
+    if fp4:
+        assert w % 2 == 0
+
+    if sf is None:
+        amax = _block_amax(xf, bh, bw).clamp(min=floor)
+        qmax_t = torch.full_like(amax, qmax)
+        dq = amax / qmax_t                                   # one correctly rounded division (cast.py:151-154)
+        if round_sf:
+            # next power of two >= dq, by carrying the mantissa into the exponent (cast.py:158-161)
+            bits = (dq.view(torch.int32) + 0x007FFFFF) & 0x7F800000
+            dq_r = bits.view(torch.float32)
+            inv = torch.where(dq_r == 0, torch.zeros_like(dq_r), 1.0 / dq_r)
+        else:
+            bits = dq.view(torch.int32)
+            inv = torch.where(bits == 0, torch.zeros_like(dq), qmax_t / amax)   # cast.py:163-164
+    else:
+        assert not use_packed_ue8m0 and not use_tma_aligned_col_major_sf
+        assert sf.ndim == 2 and tuple(sf.shape) == (nm, nk), f'scale shape {tuple(sf.shape)} != {(nm, nk)}'
+        inv = sf.reciprocal()                                # cast.py:165-170
+
+    q = xf * _expand_blocks(inv, bh, bw, h, w)
+
+    if fp4:
+        nib = encode_e2m1(q).view(h, w // 2, 2)
+        codes = (nib[..., 0] | (nib[..., 1] << 4)).view(torch.int8)     # cast.py:192-196
+    else:
+        codes = q.clamp(-qmax, qmax).to(code_dtype)                      # cast.py:188-190
+
+    if sf is not None:
+        return codes
+    return codes, _format_sf(bits, use_tma_aligned_col_major_sf, use_packed_ue8m0)
+
+
+def swiglu_forward(
+    x: torch.Tensor,
+    pos_to_token_topk: Optional[torch.Tensor] = None,
+    topk_weights: Optional[torch.Tensor] = None,
+    swiglu_clamp_value: Optional[float] = None,
+    clamped_count: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """fp32 ``silu(x[:, :H]) * x[:, H:]`` with optional clamp, clamp counters and per-row routing
+    weight; padding rows (``pos_to_token_topk < 0``) get weight 0.
+
+    Same arguments and results as ``tile_kernels.torch.swiglu_forward``
+    (tile_kernels/torch/swiglu.py:9-88); the operation order ``g / (1 + exp(-g)) * u * w`` is kept
+    because it fixes the fp32 roundings.
+    """
+    assert x.dim() == 2 and x.is_contiguous()
+    assert x.dtype in (torch.bfloat16, torch.float32)
+    rows, two_h = x.shape
+    assert two_h % 2 == 0
+    hid = two_h // 2
+    xf = x.to(torch.float32)
+    gate, up = xf[:, :hid], xf[:, hid:]
+
+    if swiglu_clamp_value is not None:
+        c = swiglu_clamp_value
+        if clamped_count is not None:   # counted before clamping, over every row (swiglu.py:66-70)
+            clamped_count += torch.stack(((gate > c).sum(), (up > c).sum(), (up < -c).sum())).to(clamped_count.dtype)
+        gate = gate.clamp(max=c)
+        up = up.clamp(min=-c, max=c)
+
+    out = gate / (1.0 + torch.exp(-gate)) * up
+
+    if pos_to_token_topk is not None:
+        assert pos_to_token_topk.dim() == 1 and pos_to_token_topk.shape[0] == rows
+        assert topk_weights is not None and topk_weights.dim() == 2
+        flat_w = topk_weights.reshape(-1).to(torch.float32)
+        live = pos_to_token_topk >= 0
+        w = torch.zeros(rows, dtype=torch.float32)
+        w[live] = flat_w[pos_to_token_topk[live].long()]
+        out = out * w[:, None]
+    return out
+
+
+def swiglu_forward_and_per_token_cast(
+    x: torch.Tensor,
+    fmt: str,
+    num_per_channels: int,
+    pos_to_token_topk: Optional[torch.Tensor] = None,
+    topk_weights: Optional[torch.Tensor] = None,
+    pos_to_expert: Optional[torch.Tensor] = None,
+    use_tma_aligned_col_major_sf: bool = False,
+    round_sf: bool = False,
+    use_packed_ue8m0: bool = False,
+    swiglu_clamp_value: Optional[float] = None,
+    clamped_count: Optional[torch.Tensor] = None,
+    sf_clamp_min: Optional[float] = None,
+):
+    """Composition the reference's own test uses as ground truth for the fused op
+    (tests/quant/test_swiglu_forward_and_per_token_cast.py:91-128): SwiGLU, zero the rows whose
+    ``pos_to_expert`` is -1, per-token cast, then codes and scales of those rows forced to zero.
+
+    Returns ``(codes, scales)`` with masked rows zeroed, i.e. what the device op must produce.
+    """
+    v = swiglu_forward(x, pos_to_token_topk, topk_weights, swiglu_clamp_value, clamped_count)
+    dead = None
+    if pos_to_expert is not None:
+        dead = (pos_to_expert < 0)[:, None]
+        v = v.masked_fill(dead, 0)
+    codes, sf = cast(v, fmt, (1, num_per_channels), round_sf=round_sf,
+                     use_tma_aligned_col_major_sf=use_tma_aligned_col_major_sf,
+                     use_packed_ue8m0=use_packed_ue8m0, amax_floor=sf_clamp_min)
+    if dead is not None:
+        codes.view(torch.uint8).masked_fill_(dead, 0)
+        sf.masked_fill_(dead, 0)          # in place: keeps the column-major strides
+    return codes, sf
