@@ -1,0 +1,136 @@
+/*
+ * tk_quant.h -- C ABI of libtk_quant.so: FP8 E4M3 / FP4 E2M1 block-scaled casts and the fused
+ * SwiGLU + per-token FP8 quantisation for AMD MI355X (gfx950).
+ *
+ * The reference exposes this path as Python functions only (there is no FFI in it); each entry
+ * point below is what a binding for one of those functions would call, and names the function
+ * it stands behind.
+ *
+ * Conventions (all entry points):
+ *   - plain pointers and sizes; every data pointer is DEVICE memory owned by the caller;
+ *   - the call validates its arguments on the host, enqueues kernels on `stream` (a hipStream_t,
+ *     NULL = the default stream) and returns without synchronising;
+ *   - it never allocates, frees or copies memory;
+ *   - return value: 0 = enqueued, < 0 = an argument was rejected and nothing was launched
+ *     (tk_status below), > 0 = a hipError_t reported by the launch;
+ *   - M == 0 (R == 0) is valid and launches nothing;
+ *   - every tk_check_* twin runs the same validation and launches nothing, so error handling can
+ *     be exercised on a machine without a GPU.
+ *
+ * Scale-factor ("sf") storage, selected by `sf_layout`; (m, k) is the block's row / column index,
+ * nm x nk the number of blocks:
+ *   TK_SF_ROW_F32    fp32, element (m, k) at sf[m * sf_ld + k]
+ *   TK_SF_COL_F32    fp32, element (m, k) at sf[k * sf_ld + m]         (sf_ld >= nm)
+ *   TK_SF_COL_UE8M0  one biased-exponent byte per block, at
+ *                    ((uint8_t*)sf)[(k / 4) * sf_ld + 4 * m + (k % 4)]  (sf_ld in BYTES, >= 4 * nm);
+ *                    needs round_sf = 1.  In cast modes the bytes of a partly filled last word
+ *                    (k >= nk) are written as 0.
+ * (reference: get_sf_shape / store_sf / load_sf, tile_kernels/quant/common.py:130-138, 219-244).
+ */
+#ifndef TK_QUANT_H
+#define TK_QUANT_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TK_QUANT_VERSION 100 /* major*10000 + minor*100 + patch */
+
+enum tk_dtype { TK_BF16 = 0, TK_F32 = 1 };
+enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1 };
+enum tk_sf_layout { TK_SF_ROW_F32 = 0, TK_SF_COL_F32 = 1, TK_SF_COL_UE8M0 = 2 };
+enum tk_mode {
+    TK_CAST_AND_SF = 0, /* write codes and scales                                  */
+    TK_SF_ONLY = 1,     /* write scales only (`out` may be NULL)                   */
+    TK_CAST_GIVEN_SF = 2 /* read scales from `sf`, write codes (quant = x * (1/sf), clamped) */
+};
+
+enum tk_status {
+    TK_OK = 0,
+    TK_ERR_NULL_POINTER = -1,
+    TK_ERR_BAD_SHAPE = -2,    /* negative size, K not a multiple of what the format needs, ... */
+    TK_ERR_BAD_DTYPE = -3,
+    TK_ERR_BAD_FORMAT = -4,
+    TK_ERR_BAD_GROUP = -5,    /* group / block size not supported                          */
+    TK_ERR_BAD_LAYOUT = -6,   /* sf_layout unknown or not allowed with this mode / round_sf */
+    TK_ERR_BAD_MODE = -7,
+    TK_ERR_BAD_STRIDE = -8,   /* row stride or sf_ld too small                              */
+    TK_ERR_MISALIGNED = -9,   /* pointer or stride not aligned for 16-byte vector access    */
+    TK_ERR_TOO_LARGE = -10,   /* more than 2^31-1 rows, columns or blocks                   */
+    TK_ERR_BAD_VALUE = -11    /* clamp / floor value not usable                             */
+};
+
+/*
+ * Per-token cast: every row of x[M, K] is cut into groups of `group` consecutive columns (the
+ * last one may be partial); each group gets one scale.
+ *   amax = max(max|x|, floor)   floor = 1e-4 (E4M3) or 6*2^-126 (E2M1)
+ *   sf   = amax / QMAX          QMAX  = 448 or 6;  with round_sf: sf = 2^ceil(log2 sf)
+ *   code = cvt(x * inv)         inv = QMAX / amax, or 1 / sf with round_sf
+ * Stands behind tile_kernels.quant.per_token_cast, per_token_cast_with_sf_only and
+ * per_token_cast_with_precomputed_sf (tile_kernels/quant/per_token_cast_kernel.py:223-302).
+ *
+ *   x            bf16 or fp32, unit column stride, `x_row_stride` elements between rows
+ *   out          E4M3: M*K bytes;  E2M1: M*K/2 bytes, element 2t in the low nibble of byte t
+ *   group        16, 32, 64, 128, or K (one scale per row; needs K % 64 == 0 and TK_CAST_AND_SF)
+ *   requirements K % 8 == 0; x and x_row_stride 16-byte aligned; out 8-byte aligned
+ */
+int tk_per_token_cast(const void *x, int x_dtype, int64_t M, int64_t K, int64_t x_row_stride, void *out,
+                      void *sf, int64_t sf_ld, int fmt, int group, int sf_layout, int round_sf, int mode,
+                      void *stream);
+int tk_check_per_token_cast(const void *x, int x_dtype, int64_t M, int64_t K, int64_t x_row_stride,
+                            const void *out, const void *sf, int64_t sf_ld, int fmt, int group, int sf_layout,
+                            int round_sf, int mode);
+
+/*
+ * Per-block cast: x[M, K] contiguous is cut into bm x bk blocks (bm, bk in {32, 128}; edge blocks
+ * may be partial); one scale per block, same arithmetic as above.
+ * Stands behind tile_kernels.quant.per_block_cast, per_block_cast_with_sf_only and
+ * per_block_cast_with_precomputed_sf (tile_kernels/quant/per_block_cast_kernel.py:205-276).
+ *   requirements K % 64 == 0; x 16-byte aligned; TK_CAST_GIVEN_SF only with TK_SF_ROW_F32
+ */
+int tk_per_block_cast(const void *x, int x_dtype, int64_t M, int64_t K, void *out, void *sf, int64_t sf_ld,
+                      int fmt, int bm, int bk, int sf_layout, int round_sf, int mode, void *stream);
+int tk_check_per_block_cast(const void *x, int x_dtype, int64_t M, int64_t K, const void *out, const void *sf,
+                            int64_t sf_ld, int fmt, int bm, int bk, int sf_layout, int round_sf, int mode);
+
+/*
+ * Fused SwiGLU + per-token E4M3 quantisation of x[R, 2H] (contiguous; gate = columns [0, H),
+ * up = columns [H, 2H)):
+ *   g, u in fp32; with use_clamp: g = min(g, clamp), u = min(max(u, -clamp), clamp)
+ *   v = g / (1 + exp(-g)) * u  [* topk_weights[pos_to_token_topk[r]], 0 where the index is < 0]
+ *   then the per-token cast above over v with groups of `group` (128 or H) columns.
+ * Stands behind tile_kernels.quant.swiglu_forward_and_per_token_cast
+ * (tile_kernels/quant/swiglu_forward_and_per_token_cast_kernel.py:175-260).
+ *
+ *   sf_clamp_min        amax floor; < 0 selects the default 1e-4
+ *   pos_to_token_topk   NULL, or int32[R] index into topk_weights (flat, `num_weights` entries)
+ *   pos_to_expert       NULL, or int32[R]; rows with a negative entry are padding: their codes and
+ *                       scales are written as zeros (the reference leaves them unwritten)
+ *   clamped_count       NULL, or int64[3] incremented by {#g > clamp, #u > clamp, #u < -clamp} over
+ *                       the non-padding rows, counted before clamping (needs use_clamp)
+ *   max_blocks          <= 0: one workgroup per tile; > 0: cap on the number of workgroups, which
+ *                       then loop over tiles (the reference's num_sms knob for the counting variant)
+ *   requirements        H % 128 == 0; group == 128, or group == H with TK_SF_ROW_F32; x 16-byte aligned
+ */
+int tk_swiglu_per_token_cast(const void *x, int x_dtype, int64_t R, int64_t H, void *out, void *sf, int64_t sf_ld,
+                             int group, int sf_layout, int round_sf, float sf_clamp_min,
+                             const int32_t *pos_to_token_topk, const float *topk_weights, int64_t num_weights,
+                             const int32_t *pos_to_expert, int use_clamp, float clamp, int64_t *clamped_count,
+                             int max_blocks, void *stream);
+int tk_check_swiglu_per_token_cast(const void *x, int x_dtype, int64_t R, int64_t H, const void *out, const void *sf,
+                                   int64_t sf_ld, int group, int sf_layout, int round_sf, float sf_clamp_min,
+                                   const int32_t *pos_to_token_topk, const float *topk_weights, int64_t num_weights,
+                                   const int32_t *pos_to_expert, int use_clamp, float clamp,
+                                   const int64_t *clamped_count);
+
+/* Text for a tk_status value (or "hip error" for positive codes). Never NULL. */
+const char *tk_strerror(int status);
+/* TK_QUANT_VERSION the library was built from. */
+int tk_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TK_QUANT_H */

@@ -1,0 +1,120 @@
+"""GPU parity of the fused SwiGLU + per-token FP8 cast against the CPU oracle.
+
+Tolerance (floating point, exp/divide rounding differs between CPU and GPU): scales within 1e-6
+relative, at most 0.01 % of the codes differ and each by one E4M3 step; clamp counters and the
+zeros of padding rows are exact.  Structure follows the reference's
+tests/quant/test_swiglu_forward_and_per_token_cast.py."""
+import pytest
+import torch
+
+from oracle import torch_ref
+from tests._util import dense_bytes, fp8_code_report, packed_sf_bytes
+
+pytestmark = pytest.mark.gpu
+
+SCALE_RTOL = 1e-6
+CODE_MISMATCH_MAX = 1e-4
+
+
+def _tk():
+    import tilekernels_amd
+    return tilekernels_amd
+
+
+def check_fused(got, want, nk, packed, what=''):
+    codes, sf = got
+    codes_ref, sf_ref = want
+    assert codes.dtype == codes_ref.dtype and tuple(codes.shape) == tuple(codes_ref.shape)
+    assert sf.dtype == sf_ref.dtype and tuple(sf.shape) == tuple(sf_ref.shape), (sf.shape, sf_ref.shape)
+    if sf.numel():
+        assert sf.stride() == sf_ref.stride(), f'{what} sf stride {sf.stride()} != {sf_ref.stride()}'
+    if packed:
+        a, b = packed_sf_bytes(sf, nk), packed_sf_bytes(sf_ref, nk)
+        assert torch.equal(a, b), f'{what}: {(a != b).sum().item()} packed scale bytes differ'
+    else:
+        a = torch.empty(sf.shape).copy_(sf.cpu())
+        b = torch.empty(sf.shape).copy_(sf_ref)
+        rel = ((a - b).abs() / b.abs().clamp(min=1e-30)).max().item() if a.numel() else 0.0
+        assert rel <= SCALE_RTOL, f'{what}: scale rel err {rel}'
+        assert torch.equal(a == 0, b == 0)
+    frac, one_step = fp8_code_report(dense_bytes(codes.cpu()), dense_bytes(codes_ref))
+    assert frac <= CODE_MISMATCH_MAX and one_step, f'{what}: {frac * 100:.5f}% codes differ, one-step={one_step}'
+    return frac
+
+
+@pytest.mark.parametrize('clamp', [None, 10.0, 0.5])
+@pytest.mark.parametrize('mode', [(False, False, False), (False, True, False), (True, True, False), (True, True, True)],
+                         ids=lambda m: 'col%d-round%d-packed%d' % tuple(int(v) for v in m))
+@pytest.mark.parametrize('with_weights', [False, True])
+@pytest.mark.parametrize('with_mask', [False, True])
+@pytest.mark.parametrize('H,N', [(2048, 128), (288 * 4 + 128, 128), (1024, 1024), (3584, 128), (384, 384)])
+def test_swiglu_forward_and_per_token_cast(H, N, with_mask, with_weights, mode, clamp):
+    tk = _tk()
+    col, rnd, packed = mode
+    if N == H and col:
+        pytest.skip('one scale per row is row-major only')
+    g = torch.Generator().manual_seed(H + 7 * N + int(with_mask) + 2 * int(with_weights))
+    pe, ptt, w = tk.testing.generate_moe_layout(97, 12, 3, 16, g, drop_fraction=0.1)
+    R = pe.numel()
+    x = torch.randn((R, 2 * H), generator=g) * 2
+    x[pe < 0] = 0
+    x = x.to(torch.bfloat16)
+    count = torch.tensor([3, 1, 4], dtype=torch.int64) if (clamp is not None and N != H) else None
+    count_ref = None if count is None else count.clone()
+    kw = dict(use_tma_aligned_col_major_sf=col, round_sf=rnd, use_packed_ue8m0=packed, swiglu_clamp_value=clamp)
+    want = torch_ref.swiglu_forward_and_per_token_cast(
+        x, 'e4m3', N, ptt if with_weights else None, w if with_weights else None, pe if with_mask else None,
+        clamped_count=count_ref, **kw)
+    for num_sms in (tk.get_device_num_sms(), 7):
+        tk.set_num_sms(num_sms)
+        cg = None if count is None else count.cuda()
+        got = tk.quant.swiglu_forward_and_per_token_cast(
+            x.cuda(), 'e4m3', N, ptt.cuda() if with_weights else None, w.cuda() if with_weights else None,
+            pe.cuda() if with_mask else None, clamped_count=cg, **kw)
+        codes, sf = got
+        if not with_mask:
+            # the reference compares padding rows as zeros on both sides (they hold silu(0)*0 = 0 anyway)
+            pass
+        check_fused(got, want, H // N, packed, f'num_sms={num_sms}')
+        if with_mask:
+            dead = pe < 0
+            assert torch.all(codes.cpu().view(torch.uint8)[dead] == 0)
+            assert torch.all(torch.empty(sf.shape, dtype=sf.dtype).copy_(sf.cpu())[dead] == 0)
+        if count is not None:
+            assert cg.cpu().tolist() == count_ref.tolist()
+    tk.set_num_sms(tk.get_device_num_sms())
+
+
+def test_swiglu_fp32_input_and_custom_floor():
+    tk = _tk()
+    x = torch.randn((50, 512)) * 3
+    want = torch_ref.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, sf_clamp_min=0.05)
+    got = tk.quant.swiglu_forward_and_per_token_cast(x.cuda(), 'e4m3', 128, sf_clamp_min=0.05)
+    check_fused(got, want, 2, False)
+    z = torch.zeros((4, 256), dtype=torch.bfloat16)
+    c, s = tk.quant.swiglu_forward_and_per_token_cast(z.cuda(), 'e4m3', 128, sf_clamp_min=448.0)
+    assert torch.all(s.cpu() == 1.0) and torch.all(c.cpu().view(torch.uint8) == 0)
+
+
+def test_swiglu_extreme_gate_values():
+    """exp(-g) overflow / underflow must give the oracle's zeros and identities, not NaN."""
+    tk = _tk()
+    x = torch.randn((8, 256))
+    x[:, 0] = -200.0
+    x[:, 1] = 200.0
+    x[:, 2] = -88.0
+    x[:, 3] = -1e30
+    x[:, 4] = 0.0
+    want = torch_ref.swiglu_forward_and_per_token_cast(x, 'e4m3', 128)
+    got = tk.quant.swiglu_forward_and_per_token_cast(x.cuda(), 'e4m3', 128)
+    check_fused(got, want, 1, False)
+    assert (got[0].cpu().view(torch.uint8) & 0x7F).max() < 0x7F
+
+
+def test_swiglu_empty():
+    tk = _tk()
+    x = torch.empty((0, 512), dtype=torch.bfloat16, device='cuda')
+    c, s = tk.quant.swiglu_forward_and_per_token_cast(x, 'e4m3', 128)
+    assert c.shape == (0, 256) and s.shape == (0, 2)
+    c, s = tk.quant.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, use_tma_aligned_col_major_sf=True, round_sf=True, use_packed_ue8m0=True)
+    assert c.shape == (0, 256) and s.shape == (0, 1) and s.dtype == torch.int32

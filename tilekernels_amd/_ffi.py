@@ -1,0 +1,91 @@
+"""ctypes binding of libtk_quant.so (the C ABI declared in include/tk_quant.h).
+
+There is deliberately no fallback: if the library has not been built, importing the ops raises.
+"""
+import ctypes
+import os
+
+import torch  # noqa: F401  (loads the HIP runtime the library links against before the library itself)
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, 'lib', 'libtk_quant.so')
+
+TK_BF16, TK_F32 = 0, 1
+TK_E4M3, TK_E2M1 = 0, 1
+TK_SF_ROW_F32, TK_SF_COL_F32, TK_SF_COL_UE8M0 = 0, 1, 2
+TK_CAST_AND_SF, TK_SF_ONLY, TK_CAST_GIVEN_SF = 0, 1, 2
+
+_i64, _i32, _vp, _f32 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_float
+
+# name -> (restype, argtypes); must list every symbol declared in include/tk_quant.h
+SIGNATURES = {
+    'tk_per_token_cast': (_i32, [_vp, _i32, _i64, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
+    'tk_check_per_token_cast': (_i32, [_vp, _i32, _i64, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32]),
+    'tk_per_block_cast': (_i32, [_vp, _i32, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
+    'tk_check_per_block_cast': (_i32, [_vp, _i32, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _i32]),
+    'tk_swiglu_per_token_cast': (_i32, [_vp, _i32, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _f32, _vp, _vp, _i64,
+                                        _vp, _i32, _f32, _vp, _i32, _vp]),
+    'tk_check_swiglu_per_token_cast': (_i32, [_vp, _i32, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _f32, _vp, _vp,
+                                              _i64, _vp, _i32, _f32, _vp]),
+    'tk_strerror': (ctypes.c_char_p, [_i32]),
+    'tk_version': (_i32, []),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once; raises if it has not been built (python -m tilekernels_amd.build)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f'{LIB_PATH} not found: build it with `python -m tilekernels_amd.build` '
+                '(hipcc, gfx950). tilekernels_amd has no CPU or PyTorch fallback.')
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+class TkError(RuntimeError):
+    pass
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        msg = load().tk_strerror(status).decode()
+        raise TkError(f'{what}: {msg} (status {status})')
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return TK_BF16
+    if t.dtype == torch.float32:
+        return TK_F32
+    raise AssertionError(f'unsupported input dtype {t.dtype}')
+
+
+def ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def current_stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_gpu(*tensors) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise TkError('tilekernels_amd runs on the GPU only (got a CPU tensor); there is no CPU path')
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise TkError(f'tensors on different devices: {dev} and {t.device}')
+    return dev

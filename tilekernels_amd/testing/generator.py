@@ -1,0 +1,88 @@
+"""Shape grids and synthetic inputs for the parity tests and the benchmark."""
+import os
+
+import torch
+
+from ..utils import align
+
+
+def _full_test() -> bool:
+    return os.getenv('TK_FULL_TEST') in ('1', 'true', 'True')
+
+
+def generate_num_tokens(alignment: int = 1, is_benchmark: bool = False):
+    """Token counts of the reference's grid (tile_kernels/testing/generator.py:10-17)."""
+    sizes = [4001, 8001]
+    if _full_test() and not is_benchmark:
+        sizes = [0] + sizes
+    return [align(n, alignment) for n in sizes]
+
+
+def generate_hidden_sizes(alignment: int = 64):
+    return [h for h in (576, 2048, 2560, 3072, 4096, 6144, 7168) if h % alignment == 0]
+
+
+def generate_moe_layout(num_tokens: int, num_experts: int, num_topk: int, alignment: int, generator: torch.Generator,
+                        drop_fraction: float = 0.0):
+    """Expert-major expanded layout of a top-k routed batch, built on the CPU.
+
+    Every (token, k) pair whose expert is >= 0 gets one row; rows are grouped by expert and every
+    expert's segment is padded to a multiple of ``alignment`` rows.  Same contract as the
+    reference's fused mapping (tile_kernels/moe/get_fused_mapping_kernel.py:166-250):
+
+      pos_to_expert[R]      expert of the row, -1 for padding
+      pos_to_token_topk[R]  token * num_topk + k of the row, -1 for padding
+      topk_weights[T, k]    softmax probabilities of the chosen experts (fp32)
+    """
+    logits = torch.randn((num_tokens, num_experts), generator=generator)
+    prob = torch.softmax(logits, dim=-1)
+    topk_w, topk_idx = torch.topk(prob, num_topk, dim=-1)
+    if drop_fraction > 0:
+        drop = torch.rand(topk_idx.shape, generator=generator) < drop_fraction
+        topk_idx = topk_idx.masked_fill(drop, -1)
+    flat = topk_idx.reshape(-1)
+    order = torch.argsort(torch.where(flat < 0, num_experts, flat), stable=True)
+    order = order[flat[order] >= 0]
+    experts = flat[order]
+    counts = torch.bincount(experts, minlength=num_experts)
+    padded = (counts + alignment - 1) // alignment * alignment
+    seg_start = torch.cumsum(padded, 0) - padded
+    rank_in_expert = torch.arange(order.numel()) - (torch.cumsum(counts, 0) - counts)[experts]
+    pos = seg_start[experts] + rank_in_expert
+    R = int(padded.sum())
+    pos_to_expert = torch.full((R,), -1, dtype=torch.int32)
+    pos_to_token_topk = torch.full((R,), -1, dtype=torch.int32)
+    pos_to_expert[pos] = experts.to(torch.int32)
+    pos_to_token_topk[pos] = order.to(torch.int32)
+    return pos_to_expert, pos_to_token_topk, topk_w.to(torch.float32).contiguous()
+
+
+def make_baseline_input(cfg: int, scale_rows: float = 1.0):
+    """Seeded CPU input of benchmark configuration ``cfg`` (1..5); ``scale_rows`` < 1 shrinks the
+    row count for quick checks.  Returns a dict with ``x`` (bf16) and, for cfg 4, the MoE layout."""
+    g = torch.Generator().manual_seed(1000 + cfg)
+    rows = lambda n: max(1, int(n * scale_rows))
+    if cfg == 1:      # activations with 0.1 % outliers x100
+        x = torch.randn((rows(4096), 7168), generator=g)
+        x[torch.rand(x.shape, generator=g) < 0.001] *= 100
+        return {'x': x.to(torch.bfloat16)}
+    if cfg == 2:      # weights N(0, 0.02) with 16 rows x50
+        m = rows(7168)
+        w = 0.02 * torch.randn((m, 2048), generator=g)
+        w[torch.randperm(m, generator=g)[: min(16, m)]] *= 50
+        return {'x': w.to(torch.bfloat16)}
+    if cfg == 3:
+        return {'x': torch.randn((rows(8192), 4096), generator=g).to(torch.bfloat16)}
+    if cfg == 4:
+        pe, ptt, w = generate_moe_layout(rows(4096), 256, 8, 128, g)
+        x = torch.randn((pe.numel(), 4096), generator=g)
+        x[pe < 0] = 0
+        return {'x': x.to(torch.bfloat16), 'pos_to_expert': pe, 'pos_to_token_topk': ptt, 'topk_weights': w}
+    if cfg == 5:      # Student-t, 4 degrees of freedom
+        m = rows(16384)
+        z = torch.randn((m, 7168), generator=g)
+        chi = torch.zeros_like(z)
+        for _ in range(4):
+            chi += torch.randn((m, 7168), generator=g) ** 2
+        return {'x': (z / torch.sqrt(chi / 4)).to(torch.bfloat16)}
+    raise ValueError(cfg)
