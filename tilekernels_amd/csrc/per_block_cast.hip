@@ -31,9 +31,7 @@ __global__ __launch_bounds__(kThreads) void per_block_cast_kernel(const PerBlock
     constexpr int IPB = BM / 16;                                     // of which per scale block
     __shared__ uint32_t amax_lds[SUBM][SUBK];
 
-    const int tile = xcd_tile_index(p.tiles_m * p.tiles_k);
-    if (tile < 0) return;
-    const int tile_m = tile / p.tiles_k, tile_k = tile - tile_m * p.tiles_k;
+    const int tile_m = blockIdx.x / p.tiles_k, tile_k = blockIdx.x - tile_m * p.tiles_k;
 
     const int t = threadIdx.x >> 4, c = threadIdx.x & 15;
     const int col = tile_k * kBlockTile + c * 8;
@@ -70,12 +68,12 @@ __global__ __launch_bounds__(kThreads) void per_block_cast_kernel(const PerBlock
         __syncthreads();
 #pragma unroll
         for (int b = 0; b < SUBM; ++b)
-            inv[b] = make_scale(u2f(amax_lds[b][bj]), Fmt<FMT>::floor_, Fmt<FMT>::qmax, p.round_sf != 0).inv;
+            inv[b] = make_scale<Fmt<FMT>::qmax>(u2f(amax_lds[b][bj]), Fmt<FMT>::floor_, p.round_sf != 0).inv;
         if (threadIdx.x < SUBM * SUBK) {
             const int b = threadIdx.x / SUBK, j = threadIdx.x % SUBK;
             const int m = tile_m * SUBM + b, k = tile_k * SUBK + j;
             if (m < p.sf.nm && k < p.sf.nk)
-                sf_store(p.sf, m, k, make_scale(u2f(amax_lds[b][j]), Fmt<FMT>::floor_, Fmt<FMT>::qmax, p.round_sf != 0));
+                sf_store(p.sf, m, k, make_scale<Fmt<FMT>::qmax>(u2f(amax_lds[b][j]), Fmt<FMT>::floor_, p.round_sf != 0));
         }
     } else {
 #pragma unroll
@@ -103,7 +101,7 @@ __global__ __launch_bounds__(kThreads) void per_block_cast_kernel(const PerBlock
 template <typename InT, int FMT>
 static hipError_t launch_per_block(const PerBlockParams &p, int bm, int bk, hipStream_t stream) {
     const int total = p.tiles_m * p.tiles_k;
-    const dim3 grid(kNumXcd * ((total + kNumXcd - 1) / kNumXcd)), block(kThreads);
+    const dim3 grid((unsigned)total), block(kThreads);
     if (bm == 128 && bk == 128) hipLaunchKernelGGL((per_block_cast_kernel<InT, FMT, 128, 128>), grid, block, 0, stream, p);
     else if (bm == 32 && bk == 32) hipLaunchKernelGGL((per_block_cast_kernel<InT, FMT, 32, 32>), grid, block, 0, stream, p);
     else if (bm == 128 && bk == 32) hipLaunchKernelGGL((per_block_cast_kernel<InT, FMT, 128, 32>), grid, block, 0, stream, p);

@@ -1,14 +1,18 @@
 // Per-token (1 x G) block-scaled cast to E4M3 / E2M1 for gfx950.
 //
-// Work decomposition: a workgroup of 4 waves owns a tile of 16 rows x 512 columns.  Each wave
-// takes 4 rows; in every row its 64 lanes cover 512 consecutive elements with one 16-byte (bf16)
-// or two 16-byte (fp32) loads per lane, all four rows' loads issued before the first use.  A group
-// of G elements therefore lives in G/8 neighbouring lanes of one DPP row and its amax needs no LDS.
-// Row-major scales are stored straight from the group's first lane; column-major layouts are
-// staged in LDS and written out transposed so that 16 lanes fill one 64-byte segment.
+// Work decomposition: a workgroup of 4 waves owns a tile of 4*RPW rows x 512 columns.  Each wave
+// takes RPW rows; in every row its 64 lanes cover 512 consecutive elements with one 16-byte (bf16)
+// or two 16-byte (fp32) streaming loads per lane, all rows' loads issued before the first use.  A
+// group of G elements therefore lives in G/8 neighbouring lanes of one DPP row and its amax needs
+// no LDS.  The divisions that turn an amax into a scale are shared out over the lanes of a group
+// (one row each) instead of being repeated by all of them.  Row-major scales are stored straight
+// from the lanes that computed them; column-major layouts are staged in LDS and written out
+// transposed so that neighbouring lanes fill one contiguous segment.
 //
 // Reference semantics: tile_kernels/quant/per_token_cast_kernel.py:65-154 (plain-tensor branch),
 // tile_kernels/quant/common.py:196-244.
+#include <stdlib.h>
+
 #include "tk_device.hpp"
 #include "tk_host.hpp"
 
@@ -20,69 +24,88 @@ struct PerTokenParams {
     SfRef sf;
     int64_t x_ld;     // elements between rows of x
     int M, K;
-    int tiles_m, tiles_k;
+    int tiles_k;
     int round_sf, mode;
 };
 
-template <typename InT, int G, int FMT>
+// Tile shapes (RPW = rows per wave):
+//   WIDE  (row-major scales):      RPW rows x 2048 columns, the 4 waves side by side on the same rows;
+//         the tile's scales are RPW contiguous runs, staged in LDS and stored as whole segments
+//   !WIDE (column-major layouts):  4*RPW rows x 512 columns, the 4 waves stacked; the staged scales
+//         are stored transposed, 4*RPW rows per contiguous segment
+// FULL: the tile grid covers the matrix exactly, so no bounds checks are compiled in.
+template <typename InT, int G, int FMT, int RPW, bool WIDE, bool FULL>
 __global__ __launch_bounds__(kThreads) void per_token_cast_kernel(const PerTokenParams p) {
     constexpr int LPG = G / 8;            // lanes per group
     constexpr int GPS = kStripCols / G;   // groups per 512-column strip
-    constexpr int RPW = kTileRows / 4;    // rows per wave
-    __shared__ uint32_t stage[kTileRows][GPS];
+    constexpr int ROWS = WIDE ? RPW : kWaves * RPW;       // rows per tile
+    constexpr int SGPR = WIDE ? kWaves * GPS : GPS;       // staged groups per row
+    using RS = RowScales<Fmt<FMT>::qmax, RPW, LPG>;
+    __shared__ uint32_t stage[ROWS][SGPR];
 
-    const int tile = xcd_tile_index(p.tiles_m * p.tiles_k);
-    if (tile < 0) return;
-    const int tile_m = tile / p.tiles_k, tile_k = tile - tile_m * p.tiles_k;
-
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int col = tile_k * kStripCols + lane * 8;
+    const int tile_m = blockIdx.x / p.tiles_k, tile_k = blockIdx.x - tile_m * p.tiles_k;
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const int strip = WIDE ? tile_k * kWaves + wave : tile_k;
+    const int col = strip * kStripCols + lane * 8;
     const int g_in_strip = lane / LPG;
-    const int kgrp = tile_k * GPS + g_in_strip;
-    const bool col_ok = col < p.K;
-    const bool leader = (lane % LPG) == 0;
-    const int row0 = tile_m * kTileRows + wave * RPW;
+    const int kgrp = strip * GPS + g_in_strip;
+    const bool col_ok = FULL || col < p.K;
+    const int srow = WIDE ? 0 : wave * RPW;                // first staged row of this wave
+    const int row0 = tile_m * ROWS + srow;
     const int64_t out_ld = FMT == TK_E4M3 ? p.K : p.K / 2;
-    const InT *x = reinterpret_cast<const InT *>(p.x);
+    const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * p.x_ld + col;
 
     Raw8<InT> raw[RPW];
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
-        const int row = row0 + r;
-        raw[r].load(x + (int64_t)row * p.x_ld + col, col_ok && row < p.M);
+        if (FULL) raw[r].load(x + (int64_t)r * p.x_ld);
+        else raw[r].load(x + (int64_t)r * p.x_ld, col_ok && row0 + r < p.M);
     }
 
-    const bool staged = p.sf.layout != TK_SF_ROW_F32 && p.mode != TK_CAST_GIVEN_SF;
+    float inv[RPW];
+    if (p.mode == TK_CAST_GIVEN_SF) {
 #pragma unroll
-    for (int r = 0; r < RPW; ++r) {
-        const int row = row0 + r;
-        const bool ok = col_ok && row < p.M;
-        float v[8];
-        raw[r].get(v);
-        Scale sc;
-        if (p.mode == TK_CAST_GIVEN_SF) {
-            const float s = ok ? sf_load(p.sf, row, kgrp) : 1.0f;
-            sc.inv = 1.0f / s;
-        } else {
-            const float amax = group_allmax<LPG>(absmax8(v));
-            sc = make_scale(amax, Fmt<FMT>::floor_, Fmt<FMT>::qmax, p.round_sf != 0);
-            if (leader) {
-                if (staged) {
-                    stage[wave * RPW + r][g_in_strip] = p.sf.layout == TK_SF_COL_F32 ? f2u(sc.sf) : sc.e8;
-                } else if (ok) {
-                    reinterpret_cast<float *>(p.sf.base)[(int64_t)row * p.sf.ld + kgrp] = sc.sf;
-                }
-            }
+        for (int r = 0; r < RPW; ++r) {
+            const bool ok = col_ok && (FULL || row0 + r < p.M);
+            inv[r] = 1.0f / (ok ? sf_load(p.sf, row0 + r, kgrp) : 1.0f);
         }
-        if (p.mode != TK_SF_ONLY && ok) {
-            uint8_t *out_row = p.out + (int64_t)row * out_ld;
-            if (p.mode == TK_CAST_GIVEN_SF) quantise_store8<FMT, true>(v, sc.inv, out_row, col);
-            else quantise_store8<FMT, false>(v, sc.inv, out_row, col);
+    } else {
+        float amax[RPW];
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            float v[8];
+            raw[r].get(v);
+            amax[r] = group_allmax<LPG>(absmax8(v));
+        }
+        RS rs;
+        rs.compute(amax, Fmt<FMT>::floor_, p.round_sf != 0, lane);
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) inv[r] = rs.inv[r];
+        // lane j (< A) of a group computed the scale of row c*A + j
+        const int own = lane % LPG;
+        if (own < RS::A) {
+#pragma unroll
+            for (int c = 0; c < RS::NC; ++c)
+                stage[srow + c * RS::A + own][(WIDE ? wave * GPS : 0) + g_in_strip] =
+                    p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
         }
     }
-    if (staged) {
+    if (p.mode != TK_SF_ONLY) {
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            if (col_ok && (FULL || row0 + r < p.M)) {
+                float v[8];
+                raw[r].get(v);
+                uint8_t *out_row = p.out + (int64_t)(row0 + r) * out_ld;
+                if (p.mode == TK_CAST_GIVEN_SF) quantise_store8<FMT, true>(v, inv[r], out_row, col);
+                else quantise_store8<FMT, false>(v, inv[r], out_row, col);
+            }
+        }
+    }
+    if (p.mode != TK_CAST_GIVEN_SF) {
         __syncthreads();
-        sf_store_tile_colmajor<GPS>(p.sf, stage, tile_m * kTileRows, tile_k * GPS);
+        if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
+        else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
     }
 }
 
@@ -97,7 +120,7 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(const PerT
     float amax = 0.0f;
     for (int col = threadIdx.x * 8; col < p.K; col += kThreads * 8) {
         Raw8<InT> raw;
-        raw.load(x + col, true);
+        raw.load_cached(x + col);
         float v[8];
         raw.get(v);
         amax = __builtin_fmaxf(amax, absmax8(v));
@@ -108,32 +131,69 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(const PerT
     uint32_t m = 0;
 #pragma unroll
     for (int i = 0; i < kThreads / 16; ++i) m = umax(m, part[i]);
-    const Scale sc = make_scale(u2f(m), Fmt<FMT>::floor_, Fmt<FMT>::qmax, p.round_sf != 0);
+    const Scale sc = make_scale<Fmt<FMT>::qmax>(u2f(m), Fmt<FMT>::floor_, p.round_sf != 0);
     if (threadIdx.x == 0) sf_store(p.sf, row, 0, sc);
     const int64_t out_ld = FMT == TK_E4M3 ? p.K : p.K / 2;
     uint8_t *out_row = p.out + (int64_t)row * out_ld;
     for (int col = threadIdx.x * 8; col < p.K; col += kThreads * 8) {
         Raw8<InT> raw;
-        raw.load(x + col, true);
+        raw.load(x + col);
         float v[8];
         raw.get(v);
         quantise_store8<FMT, false>(v, sc.inv, out_row, col);
     }
 }
 
+// rows per wave; 1, 2 or 4 (TK_PT_RPW overrides the default for tuning runs)
+static int per_token_rpw() {
+    static const int v = [] {
+        const char *e = getenv("TK_PT_RPW");
+        const int r = e ? atoi(e) : 2;
+        return (r == 1 || r == 2 || r == 4) ? r : 2;
+    }();
+    return v;
+}
+
+template <typename InT, int G, int FMT, int RPW, bool WIDE>
+static void launch_per_token_4(PerTokenParams &p, hipStream_t stream) {
+    constexpr int ROWS = WIDE ? RPW : kWaves * RPW;
+    constexpr int COLS = WIDE ? kWaves * kStripCols : kStripCols;
+    const int tiles_m = (p.M + ROWS - 1) / ROWS;
+    p.tiles_k = (p.K + COLS - 1) / COLS;
+    const dim3 grid((unsigned)(tiles_m * p.tiles_k)), block(kThreads);
+    if (p.M % ROWS == 0 && p.K % COLS == 0)
+        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, true>), grid, block, 0, stream, p);
+    else
+        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, false>), grid, block, 0, stream, p);
+}
+
+template <typename InT, int G, int FMT, int RPW>
+static void launch_per_token_3(PerTokenParams &p, hipStream_t stream) {
+    // a caller-supplied scale tensor is only read, so either tile shape does
+    if (p.sf.layout == TK_SF_ROW_F32) launch_per_token_4<InT, G, FMT, RPW, true>(p, stream);
+    else launch_per_token_4<InT, G, FMT, RPW, false>(p, stream);
+}
+
+template <typename InT, int G, int FMT>
+static void launch_per_token_2(PerTokenParams &p, hipStream_t stream) {
+    switch (per_token_rpw()) {
+        case 1: launch_per_token_3<InT, G, FMT, 1>(p, stream); break;
+        case 4: launch_per_token_3<InT, G, FMT, 4>(p, stream); break;
+        default: launch_per_token_3<InT, G, FMT, 2>(p, stream); break;
+    }
+}
+
 template <typename InT, int FMT>
-static hipError_t launch_per_token(const PerTokenParams &p, int group, hipStream_t stream) {
+static hipError_t launch_per_token(PerTokenParams &p, int group, hipStream_t stream) {
     if (group == p.K && group != 16 && group != 32 && group != 64 && group != 128) {
         hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT>), dim3(p.M), dim3(kThreads), 0, stream, p);
         return hipGetLastError();
     }
-    const int total = p.tiles_m * p.tiles_k;
-    const dim3 grid(kNumXcd * ((total + kNumXcd - 1) / kNumXcd));
     switch (group) {
-        case 16: hipLaunchKernelGGL((per_token_cast_kernel<InT, 16, FMT>), grid, dim3(kThreads), 0, stream, p); break;
-        case 32: hipLaunchKernelGGL((per_token_cast_kernel<InT, 32, FMT>), grid, dim3(kThreads), 0, stream, p); break;
-        case 64: hipLaunchKernelGGL((per_token_cast_kernel<InT, 64, FMT>), grid, dim3(kThreads), 0, stream, p); break;
-        default: hipLaunchKernelGGL((per_token_cast_kernel<InT, 128, FMT>), grid, dim3(kThreads), 0, stream, p); break;
+        case 16: launch_per_token_2<InT, 16, FMT>(p, stream); break;
+        case 32: launch_per_token_2<InT, 32, FMT>(p, stream); break;
+        case 64: launch_per_token_2<InT, 64, FMT>(p, stream); break;
+        default: launch_per_token_2<InT, 128, FMT>(p, stream); break;
     }
     return hipGetLastError();
 }
@@ -168,6 +228,7 @@ extern "C" int tk_check_per_token_cast(const void *x, int x_dtype, int64_t M, in
     if (!aligned_to(sf, 4)) return TK_ERR_MISALIGNED;
     const int64_t nk = (K + group - 1) / group;
     if (M * nk > INT32_MAX) return TK_ERR_TOO_LARGE;
+    if (((M + 3) / 4) * ((K + kStripCols - 1) / kStripCols) > INT32_MAX) return TK_ERR_TOO_LARGE;   // tile count
     const int64_t need = sf_layout == TK_SF_ROW_F32 ? nk : (sf_layout == TK_SF_COL_F32 ? M : 4 * M);
     if (sf_ld < need) return TK_ERR_BAD_STRIDE;
     if (sf_layout == TK_SF_COL_UE8M0 && sf_ld % 4 != 0) return TK_ERR_MISALIGNED;
@@ -187,11 +248,9 @@ extern "C" int tk_per_token_cast(const void *x, int x_dtype, int64_t M, int64_t 
     p.x_ld = x_row_stride;
     p.M = (int)M;
     p.K = (int)K;
-    p.tiles_m = (int)((M + kTileRows - 1) / kTileRows);
     p.tiles_k = (int)((K + kStripCols - 1) / kStripCols);
     p.round_sf = round_sf;
     p.mode = mode;
-    if ((int64_t)p.tiles_m * p.tiles_k > INT32_MAX - 8) return TK_ERR_TOO_LARGE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e;
     if (x_dtype == TK_BF16)

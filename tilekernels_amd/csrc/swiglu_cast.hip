@@ -28,41 +28,59 @@ struct SwigluParams {
     int R, H;
     int tiles_m, tiles_k;
     int round_sf;
-    int persistent;      // 1: workgroups stride over tiles by gridDim.x
     float floor_;        // amax lower clamp
     float clamp;
 };
 
-// Math variants for silu(g) = g / (1 + exp(-g)):
-//   0  v_exp_f32 on g * -log2(e), v_rcp_f32: ~12 issue slots per element, a few ulp
-//   1  libm-grade expf and an IEEE-rounded division: closest to the CPU evaluation, most ALU work
-//   2  v_exp_f32 with a two-term argument and an fma-corrected quotient: ~1.5 ulp
-template <int MATH> __device__ __forceinline__ float silu_mul(float g, float u) {
-    if (MATH == 1) {
-        const float e = expf(-g);
-        const float d = 1.0f + e;
-        return g / d * u;
-    } else if (MATH == 0) {
-        const float e = __builtin_amdgcn_exp2f(g * -1.4426950408889634f);
-        const float d = 1.0f + e;
-        return g * __builtin_amdgcn_rcpf(d) * u;
-    } else {
-        // -g * log2(e) as hi + lo, so that the rounding of the product does not reach the result
-        const float nh = -1.4426950216293335f;        // float(-log2 e)
-        const float nl = -1.9259629911266175e-8f;     // -log2 e - nh
-        const float tp = g * nh;
-        const float tl = __builtin_fmaf(g, nl, __builtin_fmaf(g, nh, -tp));
-        // exp(-g) overflows for g < -88.7; capping the exponent keeps e and d finite, so the
-        // corrected quotient below underflows to -0 / a negligible value instead of inf * 0
-        const float th = __builtin_fminf(tp, 127.0f);
-        float e = __builtin_amdgcn_exp2f(th);
-        e = __builtin_fmaf(e, tl * 0.6931471805599453f, e);
-        const float d = 1.0f + e;
-        const float r = __builtin_amdgcn_rcpf(d);
-        const float q0 = g * r;
-        const float q = __builtin_fmaf(__builtin_fmaf(-d, q0, g), r, q0);
-        return q * u;
-    }
+// silu(g) * u = g / (1 + exp(-g)) * u in fp32, built on v_exp_f32 / v_rcp_f32 (about 1 ulp each).
+// The reference's CPU evaluation (vectorised exp, IEEE division) is itself only faithful to about
+// 1 ulp in exp, so bit equality is not defined for this op; what can be matched is everything after
+// the exp: 1 + e is one IEEE addition, the quotient is corrected to (almost always) the IEEE
+// quotient, and the two products are single roundings in the reference's order.
+//
+// exp(-g) = 2^(g * -log2 e).  Rounding that product would put |g|*2^-24 of absolute error into the
+// exponent, so the constant is split into hi + lo and the lo part is applied to first order:
+// 2^(g*hi + g*lo) = 2^(g*hi) * (1 + g*lo*ln 2).
+//   bf16 input: hi keeps 15 significant bits, so g*hi is exact for an 8-bit significand
+//   fp32 input: the rounding error of g*hi is recovered with an fma and joins the lo term
+// The gate is capped at -88 inside the exponential only (the CPU's exp overflows to inf at -88.7 and
+// its quotient becomes -0): e and d then stay finite, the reciprocal underflows and the corrected
+// quotient is -0 or a value below 1e-36, never inf * 0.
+#ifndef TK_SWIGLU_NEWTON
+#define TK_SWIGLU_NEWTON 1
+#endif
+
+// g / d from r ~ 1/d: one Newton step on the quotient (two fmas)
+__device__ __forceinline__ float quotient(float g, float d) {
+    const float r = __builtin_amdgcn_rcpf(d);
+    const float q0 = g * r;
+#if TK_SWIGLU_NEWTON
+    return __builtin_fmaf(__builtin_fmaf(-d, q0, g), r, q0);
+#else
+    return q0;
+#endif
+}
+
+template <typename InT> __device__ __forceinline__ float silu_mul(float g, float u);
+
+template <> __device__ __forceinline__ float silu_mul<bf16_t>(float g, float u) {
+    constexpr float nh = -1.44268798828125f;             // -log2(e) cut to 15 significant bits (0xBFB8AA00)
+    constexpr float nl_ln2 = -4.8884952e-06f;            // (-log2(e) - nh) * ln 2
+    const float gc = __builtin_fmaxf(g, -88.0f);
+    const float e0 = __builtin_amdgcn_exp2f(gc * nh);    // exact product
+    const float e = __builtin_fmaf(e0, gc * nl_ln2, e0);
+    return quotient(g, 1.0f + e) * u;
+}
+
+template <> __device__ __forceinline__ float silu_mul<float>(float g, float u) {
+    constexpr float nh = -1.4426950216293335f;           // float(-log2 e)
+    constexpr float nl = -1.9259629911266175e-8f;        // -log2 e - nh
+    const float gc = __builtin_fmaxf(g, -88.0f);
+    const float th = gc * nh;
+    const float tl = __builtin_fmaf(gc, nl, __builtin_fmaf(gc, nh, -th));
+    const float e0 = __builtin_amdgcn_exp2f(th);
+    const float e = __builtin_fmaf(e0, tl * 0.6931471805599453f, e0);
+    return quotient(g, 1.0f + e) * u;
 }
 
 // CLAMP: 0 none, 1 clamp, 2 clamp and count
@@ -88,86 +106,116 @@ template <int CLAMP> struct ClampCounter {
     }
 };
 
+// `row` must be wave-uniform
 __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
-    const int pos = p.pos_to_token_topk[row];
-    return (pos >= 0 && pos < p.num_weights) ? p.topk_weights[pos] : 0.0f;
+    const int pos = uniform_load(p.pos_to_token_topk + row);
+    return (pos >= 0 && pos < p.num_weights) ? uniform_load(p.topk_weights + pos) : 0.0f;
 }
 
-template <typename InT, int CLAMP, int MATH>
+// Tile shapes as in the per-token cast (RPW = rows per wave):
+//   WIDE  (row-major scales):     RPW rows x 2048 output columns, the 4 waves side by side; the tile's
+//         scales are RPW contiguous runs of 16, staged in LDS and stored as whole segments
+//   !WIDE (column-major layouts): 4*RPW rows x 512 columns, the 4 waves stacked, scales stored transposed
+// FULL: the tile grid covers the matrix exactly: no bounds checks are compiled in.
+// MASK: pos_to_expert is given.
+template <typename InT, int CLAMP, int RPW, bool WIDE, bool FULL, bool MASK>
 __global__ __launch_bounds__(kThreads) void swiglu_cast_kernel(const SwigluParams p) {
     constexpr int GPS = kStripCols / 128;   // 4 groups per strip
-    constexpr int RPW = kTileRows / 4;
-    __shared__ uint32_t stage[kTileRows][GPS];
+    constexpr int ROWS = WIDE ? RPW : kWaves * RPW;
+    constexpr int SGPR = WIDE ? kWaves * GPS : GPS;
+    using RS = RowScales<448, RPW, 16>;
+    __shared__ uint32_t stage[ROWS][SGPR];
 
     const int total = p.tiles_m * p.tiles_k;
-    int tile = p.persistent ? (int)blockIdx.x : xcd_tile_index(total);
-    const int step = p.persistent ? (int)gridDim.x : total;
-    if (tile < 0) tile = total;   // surplus workgroup: no tile, but it still reaches the counter flush
-
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const bool leader = (lane & 15) == 0;
-    const bool staged = p.sf.layout != TK_SF_ROW_F32;
-    const InT *x = reinterpret_cast<const InT *>(p.x);
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const bool has_weight = p.pos_to_token_topk != nullptr;
+    const int own = lane & 15;
+    const int srow = WIDE ? 0 : wave * RPW;
     ClampCounter<CLAMP> counter;
 
-    for (; tile < total; tile += step) {
+    for (int tile = blockIdx.x; tile < total; tile += gridDim.x) {
         const int tile_m = tile / p.tiles_k, tile_k = tile - tile_m * p.tiles_k;
-        const int col = tile_k * kStripCols + lane * 8;
-        const int kgrp = tile_k * GPS + (lane >> 4);
-        const bool col_ok = col < p.H;
-        const int row0 = tile_m * kTileRows + wave * RPW;
+        const int strip = WIDE ? tile_k * kWaves + wave : tile_k;
+        const int col = strip * kStripCols + lane * 8;
+        const bool col_ok = FULL || col < p.H;
+        const int row0 = tile_m * ROWS + srow;
+        const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * (2 * (int64_t)p.H) + col;
 
         Raw8<InT> rg[RPW], ru[RPW];
-        bool live[RPW];
+        bool live[RPW];   // wave-uniform
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
-            const int row = row0 + r;
-            live[r] = row < p.R && (p.pos_to_expert == nullptr || p.pos_to_expert[row] >= 0);
-            const InT *xr = x + (int64_t)row * (2 * (int64_t)p.H) + col;
-            rg[r].load(xr, live[r] && col_ok);
-            ru[r].load(xr + p.H, live[r] && col_ok);
+            live[r] = FULL || row0 + r < p.R;
+            if (MASK && live[r]) live[r] = uniform_load(p.pos_to_expert + row0 + r) >= 0;
+            const InT *xr = x + (int64_t)r * (2 * (int64_t)p.H);
+            if (FULL && !MASK) {
+                rg[r].load(xr);
+                ru[r].load(xr + p.H);
+            } else {
+                rg[r].load(xr, live[r] && col_ok);
+                ru[r].load(xr + p.H, live[r] && col_ok);
+            }
         }
+
+        // dead rows hold zeros, so they flow through as v = 0 and only their scale is overridden
+        float v[RPW][8], amax[RPW];
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
-            const int row = row0 + r;
-            const bool in_range = row < p.R && col_ok;
-            float g[8], u[8], v[8];
+            float g[8], u[8];
             rg[r].get(g);
             ru[r].get(u);
-            Scale sc;
-            if (live[r]) {   // wave-uniform
-                const float w = p.pos_to_token_topk ? row_weight(p, row) : 1.0f;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    if (col_ok) counter.apply(g[i], u[i], p.clamp);
-                    v[i] = silu_mul<MATH>(g[i], u[i]);
-                    if (p.pos_to_token_topk) v[i] = v[i] * w;
-                }
-                const float amax = group_allmax<16>(absmax8(v));
-                sc = make_scale(amax, p.floor_, 448.0f, p.round_sf != 0);
-            } else {
+            for (int i = 0; i < 8; ++i) {
+                counter.apply(g[i], u[i], p.clamp);
+                v[r][i] = silu_mul<InT>(g[i], u[i]);
+            }
+            if (has_weight) {
+                const float w = live[r] ? row_weight(p, row0 + r) : 0.0f;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) v[i] = 0.0f;
-                sc.sf = 0.0f; sc.inv = 0.0f; sc.e8 = 0u;
+                for (int i = 0; i < 8; ++i) v[r][i] = v[r][i] * w;
             }
-            if (leader) {
-                if (staged) stage[wave * RPW + r][lane >> 4] = p.sf.layout == TK_SF_COL_F32 ? f2u(sc.sf) : sc.e8;
-                else if (in_range) reinterpret_cast<float *>(p.sf.base)[(int64_t)row * p.sf.ld + kgrp] = sc.sf;
+            amax[r] = group_allmax<16>(absmax8(v[r]));
+        }
+        RS rs;
+        rs.compute(amax, p.floor_, p.round_sf != 0, lane);
+        if (MASK) {
+#pragma unroll
+            for (int c = 0; c < RS::NC; ++c) {
+                const int pick = lane & (RS::A - 1);
+                const bool l0 = live[c * RS::A];
+                const bool l1 = RS::A >= 2 ? live[c * RS::A + (RS::A >= 2 ? 1 : 0)] : false;
+                const bool l2 = RS::A >= 4 ? live[c * RS::A + (RS::A >= 4 ? 2 : 0)] : false;
+                const bool l3 = RS::A >= 4 ? live[c * RS::A + (RS::A >= 4 ? 3 : 0)] : false;
+                bool mine = l0;
+                if (RS::A >= 2) mine = pick == 1 ? l1 : mine;
+                if (RS::A >= 4) { mine = pick == 2 ? l2 : mine; mine = pick == 3 ? l3 : mine; }
+                if (!mine) { rs.own[c].sf = 0.0f; rs.own[c].e8 = 0u; }
             }
-            if (in_range) quantise_store8<TK_E4M3, false>(v, sc.inv, p.out + (int64_t)row * p.H, col);
+#pragma unroll
+            for (int r = 0; r < RPW; ++r) rs.inv[r] = live[r] ? rs.inv[r] : 0.0f;
         }
-        if (staged) {
-            __syncthreads();
-            sf_store_tile_colmajor<GPS>(p.sf, stage, tile_m * kTileRows, tile_k * GPS);
-            __syncthreads();   // stage is reused by the next tile
+        // lane j (< A) of a group computed the scale of row c*A + j
+        if (own < RS::A) {
+#pragma unroll
+            for (int c = 0; c < RS::NC; ++c)
+                stage[srow + c * RS::A + own][(WIDE ? wave * GPS : 0) + (lane >> 4)] =
+                    p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
         }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r)
+            if (col_ok && (FULL || row0 + r < p.R))
+                quantise_store8<TK_E4M3, false>(v[r], rs.inv[r], p.out + (int64_t)(row0 + r) * p.H, col);
+        __syncthreads();
+        if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
+        else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
+        if (gridDim.x < total) __syncthreads();   // stage is reused by the next tile
     }
     counter.flush(p.clamped_count);
 }
 
 // One scale per row (group == H): a workgroup per row, the activation is evaluated twice (amax
 // pass, then convert pass; the second read comes from L2).  Row-major scales only.
-template <typename InT, int CLAMP, int MATH>
+template <typename InT, int CLAMP>
 __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(const SwigluParams p) {
     __shared__ uint32_t part[kThreads / 16];
     const InT *xb = reinterpret_cast<const InT *>(p.x);
@@ -177,7 +225,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(const SwigluP
         uint8_t *out_row = p.out + (int64_t)row * p.H;
         float *sf_row = reinterpret_cast<float *>(p.sf.base) + (int64_t)row * p.sf.ld;
         if (!live) {
-            for (int col = threadIdx.x * 8; col < p.H; col += kThreads * 8) *reinterpret_cast<uint2 *>(out_row + col) = make_uint2(0, 0);
+            for (int col = threadIdx.x * 8; col < p.H; col += kThreads * 8) st_stream8(out_row + col, u32x2{0u, 0u});
             if (threadIdx.x == 0) sf_row[0] = 0.0f;
             continue;
         }
@@ -187,8 +235,8 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(const SwigluP
         for (int pass = 0; pass < 2; ++pass) {
             for (int col = threadIdx.x * 8; col < p.H; col += kThreads * 8) {
                 Raw8<InT> rg, ru;
-                rg.load(x + col, true);
-                ru.load(x + p.H + col, true);
+                rg.load_cached(x + col);
+                ru.load_cached(x + p.H + col);
                 float g[8], u[8], v[8];
                 rg.get(g);
                 ru.get(u);
@@ -196,7 +244,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(const SwigluP
                 for (int i = 0; i < 8; ++i) {
                     if (pass == 0) counter.apply(g[i], u[i], p.clamp);
                     else ClampCounter<(CLAMP ? 1 : 0)>().apply(g[i], u[i], p.clamp);
-                    v[i] = silu_mul<MATH>(g[i], u[i]);
+                    v[i] = silu_mul<InT>(g[i], u[i]);
                     if (p.pos_to_token_topk) v[i] = v[i] * w;
                 }
                 if (pass == 0) amax = __builtin_fmaxf(amax, absmax8(v));
@@ -210,7 +258,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(const SwigluP
                 uint32_t m = 0;
 #pragma unroll
                 for (int i = 0; i < kThreads / 16; ++i) m = umax(m, part[i]);
-                const Scale sc = make_scale(u2f(m), p.floor_, 448.0f, p.round_sf != 0);
+                const Scale sc = make_scale<448>(u2f(m), p.floor_, p.round_sf != 0);
                 inv = sc.inv;
                 if (threadIdx.x == 0) sf_row[0] = sc.sf;
             }
@@ -219,39 +267,60 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(const SwigluP
     counter.flush(p.clamped_count);
 }
 
-static int swiglu_math_variant() {
+// rows per wave of the tiled kernel; 1, 2 or 4 (TK_SWIGLU_RPW overrides the default for tuning runs)
+static int swiglu_rpw() {
     static const int v = [] {
-        const char *e = getenv("TK_SWIGLU_MATH");
-        const int m = e ? atoi(e) : 2;
-        return (m < 0 || m > 2) ? 2 : m;
+        const char *e = getenv("TK_SWIGLU_RPW");
+        const int r = e ? atoi(e) : 2;
+        return (r == 1 || r == 2 || r == 4) ? r : 2;
     }();
     return v;
 }
 
-template <typename InT, int CLAMP, int MATH>
-static hipError_t launch_swiglu_3(const SwigluParams &p, bool row_group, int max_blocks, hipStream_t stream) {
+template <typename InT, int CLAMP, int RPW, bool WIDE>
+static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t stream) {
+    constexpr int ROWS = WIDE ? RPW : kWaves * RPW;
+    constexpr int COLS = WIDE ? kWaves * kStripCols : kStripCols;
+    p.tiles_m = (p.R + ROWS - 1) / ROWS;
+    p.tiles_k = (p.H + COLS - 1) / COLS;
+    const int total = p.tiles_m * p.tiles_k;
+    const dim3 grid((unsigned)((max_blocks > 0 && max_blocks < total) ? max_blocks : total)), block(kThreads);
+    const bool full = p.R % ROWS == 0 && p.H % COLS == 0;
+    if (p.pos_to_expert) {
+        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, true, true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, false, true>), grid, block, 0, stream, p);
+    } else {
+        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, true, false>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, false, false>), grid, block, 0, stream, p);
+    }
+}
+
+template <typename InT, int CLAMP>
+static hipError_t launch_swiglu_2(SwigluParams &p, bool row_group, int max_blocks, hipStream_t stream) {
     if (row_group) {
         const int grid = max_blocks > 0 && max_blocks < p.R ? max_blocks : p.R;
-        hipLaunchKernelGGL((swiglu_rowgroup_kernel<InT, CLAMP, MATH>), dim3(grid), dim3(kThreads), 0, stream, p);
+        hipLaunchKernelGGL((swiglu_rowgroup_kernel<InT, CLAMP>), dim3(grid), dim3(kThreads), 0, stream, p);
     } else {
-        const int total = p.tiles_m * p.tiles_k;
-        const int grid = p.persistent ? max_blocks : kNumXcd * ((total + kNumXcd - 1) / kNumXcd);
-        hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, MATH>), dim3(grid), dim3(kThreads), 0, stream, p);
+        const int rpw = swiglu_rpw();
+        if (p.sf.layout == TK_SF_ROW_F32) {
+            switch (rpw) {
+                case 1: launch_swiglu_tiled<InT, CLAMP, 1, true>(p, max_blocks, stream); break;
+                case 4: launch_swiglu_tiled<InT, CLAMP, 4, true>(p, max_blocks, stream); break;
+                default: launch_swiglu_tiled<InT, CLAMP, 2, true>(p, max_blocks, stream); break;
+            }
+        } else {
+            switch (rpw) {
+                case 1: launch_swiglu_tiled<InT, CLAMP, 1, false>(p, max_blocks, stream); break;
+                case 4: launch_swiglu_tiled<InT, CLAMP, 4, false>(p, max_blocks, stream); break;
+                default: launch_swiglu_tiled<InT, CLAMP, 2, false>(p, max_blocks, stream); break;
+            }
+        }
     }
     return hipGetLastError();
 }
 
-template <typename InT, int CLAMP>
-static hipError_t launch_swiglu_2(const SwigluParams &p, bool row_group, int max_blocks, hipStream_t stream) {
-    switch (swiglu_math_variant()) {
-        case 0: return launch_swiglu_3<InT, CLAMP, 0>(p, row_group, max_blocks, stream);
-        case 1: return launch_swiglu_3<InT, CLAMP, 1>(p, row_group, max_blocks, stream);
-        default: return launch_swiglu_3<InT, CLAMP, 2>(p, row_group, max_blocks, stream);
-    }
-}
-
 template <typename InT>
-static hipError_t launch_swiglu_1(const SwigluParams &p, int clamp_mode, bool row_group, int max_blocks, hipStream_t stream) {
+static hipError_t launch_swiglu_1(SwigluParams &p, int clamp_mode, bool row_group, int max_blocks, hipStream_t stream) {
     switch (clamp_mode) {
         case 0: return launch_swiglu_2<InT, 0>(p, row_group, max_blocks, stream);
         case 1: return launch_swiglu_2<InT, 1>(p, row_group, max_blocks, stream);
@@ -289,7 +358,7 @@ extern "C" int tk_check_swiglu_per_token_cast(const void *x, int x_dtype, int64_
     const int64_t need = sf_layout == TK_SF_ROW_F32 ? nk : (sf_layout == TK_SF_COL_F32 ? R : 4 * R);
     if (sf_ld < need) return TK_ERR_BAD_STRIDE;
     if (sf_layout == TK_SF_COL_UE8M0 && sf_ld % 4 != 0) return TK_ERR_MISALIGNED;
-    const int64_t tiles = ((R + kTileRows - 1) / kTileRows) * ((H + kStripCols - 1) / kStripCols);
+    const int64_t tiles = ((R + 3) / 4) * ((H + kStripCols - 1) / kStripCols);
     if (tiles > INT32_MAX - 8) return TK_ERR_TOO_LARGE;
     return TK_OK;
 }
@@ -315,10 +384,8 @@ extern "C" int tk_swiglu_per_token_cast(const void *x, int x_dtype, int64_t R, i
     p.num_weights = num_weights;
     p.R = (int)R;
     p.H = (int)H;
-    p.tiles_m = (int)((R + kTileRows - 1) / kTileRows);
-    p.tiles_k = (int)((H + kStripCols - 1) / kStripCols);
+    p.tiles_m = p.tiles_k = 0;
     p.round_sf = round_sf;
-    p.persistent = (max_blocks > 0 && max_blocks < p.tiles_m * p.tiles_k) ? 1 : 0;
     p.floor_ = sf_clamp_min < 0.0f ? 1e-4f : sf_clamp_min;
     p.clamp = clamp;
     const int clamp_mode = use_clamp ? (clamped_count ? 2 : 1) : 0;

@@ -1,5 +1,6 @@
-// Device-side building blocks shared by the gfx950 quantisation kernels: 16-byte vector loads,
-// DPP cross-lane maxima, scale arithmetic, OCP FP8 / FP4 packing and scale-factor addressing.
+// Device-side building blocks shared by the gfx950 quantisation kernels: streaming 16-byte loads
+// and stores, DPP cross-lane maxima, scale arithmetic, OCP FP8 / FP4 packing and scale-factor
+// addressing.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -9,54 +10,84 @@
 
 namespace tk {
 
-constexpr int kTileRows = 16;     // rows of one workgroup tile (4 waves x 4 rows)
 constexpr int kStripCols = 512;   // columns one wave covers per row: 64 lanes x 8 elements
-constexpr int kThreads = 256;
-constexpr int kNumXcd = 8;        // MI355X: workgroup i is dispatched to XCD i % 8
+constexpr int kThreads = 256;     // 4 waves per workgroup
+constexpr int kWaves = kThreads / 64;
 
 struct bf16_t { uint16_t bits; };
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
 
-// ---------------------------------------------------------------------------------------------
-// Workgroup -> tile mapping.  Consecutive workgroup ids land on different XCDs (each with its own
-// L2), so tile t is handed to workgroup (t % per) * 8 + t / per ... inverted here: the workgroups
-// of one XCD walk a contiguous range of tiles, which keeps partially written scale-factor cache
-// lines inside one L2 until they are complete.
-// Launch with grid = kNumXcd * ceil(total / kNumXcd); returns -1 for the surplus workgroups.
-__device__ __forceinline__ int xcd_tile_index(int total) {
-    const int per = (total + kNumXcd - 1) / kNumXcd;
-    const int bid = blockIdx.x;
-    const int t = (bid % kNumXcd) * per + bid / kNumXcd;
-    return t < total ? t : -1;
+// Wave index as a scalar: everything derived from it (row numbers, row pointers, per-row flags)
+// then lives in SGPRs and uses scalar loads.
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
+// Load through the scalar (constant) path: for small read-only tables indexed by a wave-uniform
+// value, so that the result arrives in an SGPR and does not tie up the vector memory counter.
+template <typename T> __device__ __forceinline__ T uniform_load(const T *p) {
+    typedef const T __attribute__((address_space(4))) *const_ptr;
+    return *(const_ptr)(uintptr_t)p;
 }
 
 // ---------------------------------------------------------------------------------------------
-// Loads of 8 consecutive elements as fp32.  `ok == false` yields zeros without touching memory.
-__device__ __forceinline__ void unpack_bf16x8(const uint4 w, float (&v)[8]) {
-    v[0] = u2f(w.x << 16); v[1] = u2f(w.x & 0xFFFF0000u);
-    v[2] = u2f(w.y << 16); v[3] = u2f(w.y & 0xFFFF0000u);
-    v[4] = u2f(w.z << 16); v[5] = u2f(w.z & 0xFFFF0000u);
-    v[6] = u2f(w.w << 16); v[7] = u2f(w.w & 0xFFFF0000u);
+// Streaming memory access.  Inputs are read once and outputs written once.  Measured on MI355X for
+// the SwiGLU traffic shape (64 MiB read, 16 MiB written per call, buffers rotated past the last-
+// level cache), time per call with plain / hinted accesses:
+//     plain loads, plain stores                15.5 us
+//     non-temporal loads, plain stores         14.8 us
+//     non-temporal loads, non-temporal stores  14.2 us
+//     non-temporal loads, write-through stores 13.8 us   <- used here
+// Loads carry the `nt` bit; stores are issued at system scope (`sc0 sc1`), which writes them
+// through instead of leaving dirty lines to be flushed when the kernel ends.
+__device__ __forceinline__ u32x4 ld_stream16(const void *p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+}
+__device__ __forceinline__ void st_stream8(void *p, u32x2 v) {
+    __hip_atomic_store(reinterpret_cast<uint64_t *>(p), __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ void st_stream4(void *p, uint32_t v) {
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// 8 consecutive elements, as fp32.  `ok == false` yields zeros without touching memory.
 template <typename T> struct Raw8;
 template <> struct Raw8<bf16_t> {
-    uint4 w;
+    u32x4 w;
+    __device__ __forceinline__ void load(const bf16_t *p) { w = ld_stream16(p); }
     __device__ __forceinline__ void load(const bf16_t *p, bool ok) {
-        w = ok ? *reinterpret_cast<const uint4 *>(p) : make_uint4(0, 0, 0, 0);
+        w = u32x4{0u, 0u, 0u, 0u};
+        if (ok) w = ld_stream16(p);
     }
-    __device__ __forceinline__ void get(float (&v)[8]) const { unpack_bf16x8(w, v); }
+    // ordinary (cacheable) load, for data that is read again shortly
+    __device__ __forceinline__ void load_cached(const bf16_t *p) { w = *reinterpret_cast<const u32x4 *>(p); }
+    __device__ __forceinline__ void zero() { w = u32x4{0u, 0u, 0u, 0u}; }
+    __device__ __forceinline__ void get(float (&v)[8]) const {
+        v[0] = u2f(w.x << 16); v[1] = u2f(w.x & 0xFFFF0000u);
+        v[2] = u2f(w.y << 16); v[3] = u2f(w.y & 0xFFFF0000u);
+        v[4] = u2f(w.z << 16); v[5] = u2f(w.z & 0xFFFF0000u);
+        v[6] = u2f(w.w << 16); v[7] = u2f(w.w & 0xFFFF0000u);
+    }
 };
 template <> struct Raw8<float> {
-    float4 a, b;
+    u32x4 a, b;
+    __device__ __forceinline__ void load(const float *p) { a = ld_stream16(p); b = ld_stream16(p + 4); }
     __device__ __forceinline__ void load(const float *p, bool ok) {
-        a = ok ? *reinterpret_cast<const float4 *>(p) : make_float4(0, 0, 0, 0);
-        b = ok ? *reinterpret_cast<const float4 *>(p + 4) : make_float4(0, 0, 0, 0);
+        zero();
+        if (ok) { a = ld_stream16(p); b = ld_stream16(p + 4); }
     }
+    __device__ __forceinline__ void load_cached(const float *p) {
+        a = *reinterpret_cast<const u32x4 *>(p);
+        b = *reinterpret_cast<const u32x4 *>(p + 4);
+    }
+    __device__ __forceinline__ void zero() { a = u32x4{0u, 0u, 0u, 0u}; b = a; }
     __device__ __forceinline__ void get(float (&v)[8]) const {
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+        v[0] = u2f(a.x); v[1] = u2f(a.y); v[2] = u2f(a.z); v[3] = u2f(a.w);
+        v[4] = u2f(b.x); v[5] = u2f(b.y); v[6] = u2f(b.z); v[7] = u2f(b.w);
     }
 };
 
@@ -68,8 +99,8 @@ __device__ __forceinline__ float absmax8(const float (&v)[8]) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Cross-lane maxima on DPP (no LDS).  Operands are non-negative floats, whose order is the order
-// of their bit patterns as unsigned integers, so the steps use integer max.
+// Cross-lane operations on DPP (no LDS).  Maxima take non-negative floats, whose order is the
+// order of their bit patterns as unsigned integers, so the steps use integer max.
 template <int CTRL> __device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
 }
@@ -77,8 +108,6 @@ constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
 constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
 constexpr int kDppHalfMirror = 0x141; // lane i <-> 7-i inside each 8
 constexpr int kDppMirror = 0x140;     // lane i <-> 15-i inside each 16
-constexpr int kDppRowShl4 = 0x104;    // lane i reads lane i+4 of its 16-lane row (0 past the end)
-constexpr int kDppRowShl8 = 0x108;
 
 __device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
 
@@ -90,6 +119,14 @@ template <int LANES> __device__ __forceinline__ float group_allmax(float nonneg)
     if (LANES >= 8) v = umax(v, dpp_u32<kDppHalfMirror>(v));
     if (LANES >= 16) v = umax(v, dpp_u32<kDppMirror>(v));
     return u2f(v);
+}
+
+// value held by lane j of every aligned set of A (1, 2 or 4) lanes
+template <int A, int J> __device__ __forceinline__ float bcast_within(float v) {
+    static_assert(A == 1 || A == 2 || A == 4, "A");
+    if (A == 1) return v;
+    constexpr int ctrl = A == 4 ? J * 0x55 : (J ? 0xF5 : 0xA0);   // quad_perm [j,j,j,j] / [j,j,2+j,2+j]
+    return u2f(dpp_u32<ctrl>(f2u(v)));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -104,13 +141,25 @@ struct Scale {
     uint32_t e8;    // biased exponent of sf (UE8M0 byte), valid with round_sf
 };
 
-__device__ __forceinline__ Scale make_scale(float amax, float floor_, float qmax, bool round_sf) {
+// a / C for C in {448, 6}, correctly rounded, in three instructions: q = a*y, r = fma(-C, q, a),
+// q + r*y with y = fl(1/C).  For these two constants the result equals the IEEE quotient for EVERY
+// positive float whose quotient is a normal number (checked exhaustively over all 2^31 inputs on the
+// CPU with a correctly rounded fmaf); smaller operands take the ordinary division.
+template <int QMAX> __device__ __forceinline__ float div_by_qmax(float a) {
+    constexpr float c = (float)QMAX;
+    constexpr float y = 1.0f / c;
+    if (a < 0x1p-100f) return a / c;
+    const float q = a * y;
+    return __builtin_fmaf(__builtin_fmaf(-c, q, a), y, q);
+}
+
+template <int QMAX> __device__ __forceinline__ Scale make_scale(float amax, float floor_, bool round_sf) {
     const float a = __builtin_fmaxf(amax, floor_);
-    const float s = a / qmax;
+    const float s = div_by_qmax<QMAX>(a);
     Scale r;
     if (!round_sf) {
         r.sf = s;
-        r.inv = f2u(s) == 0u ? 0.0f : qmax / a;
+        r.inv = f2u(s) == 0u ? 0.0f : (float)QMAX / a;
         r.e8 = f2u(s) >> 23;
     } else {
         const uint32_t b = (f2u(s) + 0x007FFFFFu) & 0x7F800000u;
@@ -125,18 +174,54 @@ __device__ __forceinline__ Scale make_scale(float amax, float floor_, float qmax
 
 template <int FMT> struct Fmt;
 template <> struct Fmt<TK_E4M3> {
-    static constexpr float qmax = 448.0f;
+    static constexpr int qmax = 448;
     static constexpr float floor_ = 1e-4f;
 };
 template <> struct Fmt<TK_E2M1> {
-    static constexpr float qmax = 6.0f;
+    static constexpr int qmax = 6;
     static constexpr float floor_ = 6.0f * 0x1p-126f;
+};
+
+// Scales of RPW rows at once.  All lanes of a group already hold the group's amax of every row, so
+// instead of every lane repeating the same divisions for every row, lane i of each aligned set of
+// A lanes computes the scale of row c*A + i only and the multipliers are handed round with DPP.
+//   own[c] : scale computed by this lane, i.e. of row c*A + (lane % A)
+//   inv[r] : multiplier of row r, valid in every lane
+template <int QMAX, int RPW, int LPG> struct RowScales {
+    static constexpr int A = RPW >= 4 && LPG >= 4 ? 4 : (RPW >= 2 ? 2 : 1);
+    static constexpr int NC = RPW / A;
+    static_assert(RPW % A == 0 && LPG % A == 0, "rows per wave and lanes per group must be multiples of A");
+    Scale own[NC];
+    float inv[RPW];
+
+    __device__ __forceinline__ void compute(const float (&amax)[RPW], float floor_, bool round_sf, int lane) {
+        const int pick = lane & (A - 1);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            // all candidates are read unconditionally and chosen by value, so the array never has to
+            // be addressed dynamically
+            const float a0 = amax[c * A];
+            const float a1 = A >= 2 ? amax[c * A + (A >= 2 ? 1 : 0)] : 0.0f;
+            const float a2 = A >= 4 ? amax[c * A + (A >= 4 ? 2 : 0)] : 0.0f;
+            const float a3 = A >= 4 ? amax[c * A + (A >= 4 ? 3 : 0)] : 0.0f;
+            float a = a0;
+            if (A >= 2) a = pick == 1 ? a1 : a;
+            if (A >= 4) { a = pick == 2 ? a2 : a; a = pick == 3 ? a3 : a; }
+            own[c] = make_scale<QMAX>(a, floor_, round_sf);
+            inv[c * A] = bcast_within<A, 0>(own[c].inv);
+            if (A >= 2) inv[c * A + (A >= 2 ? 1 : 0)] = bcast_within<A, 1>(own[c].inv);
+            if (A >= 4) {
+                inv[c * A + (A >= 4 ? 2 : 0)] = bcast_within<A, 2>(own[c].inv);
+                inv[c * A + (A >= 4 ? 3 : 0)] = bcast_within<A, 3>(own[c].inv);
+            }
+        }
+    }
 };
 
 // ---------------------------------------------------------------------------------------------
 // Conversions.  v_cvt_pk_fp8_f32 on gfx950 is OCP E4M3FN round-to-nearest-even; it does not
 // saturate by itself, so inputs that may exceed 448 are clamped first (CLAMP).
-template <bool CLAMP> __device__ __forceinline__ uint2 pack_e4m3x8(const float (&q)[8]) {
+template <bool CLAMP> __device__ __forceinline__ u32x2 pack_e4m3x8(const float (&q)[8]) {
     float c[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) c[i] = CLAMP ? __builtin_amdgcn_fmed3f(q[i], -448.0f, 448.0f) : q[i];
@@ -144,7 +229,7 @@ template <bool CLAMP> __device__ __forceinline__ uint2 pack_e4m3x8(const float (
     lo = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], lo, true);
     int hi = __builtin_amdgcn_cvt_pk_fp8_f32(c[4], c[5], 0, false);
     hi = __builtin_amdgcn_cvt_pk_fp8_f32(c[6], c[7], hi, true);
-    return make_uint2((uint32_t)lo, (uint32_t)hi);
+    return u32x2{(uint32_t)lo, (uint32_t)hi};
 }
 
 // eight fp32 -> eight E2M1 nibbles in one dword, element 2t in the low nibble of byte t
@@ -163,11 +248,8 @@ __device__ __forceinline__ void quantise_store8(const float (&v)[8], float inv, 
     float q[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) q[i] = v[i] * inv;
-    if (FMT == TK_E4M3) {
-        *reinterpret_cast<uint2 *>(out_row + col) = pack_e4m3x8<CLAMP>(q);
-    } else {
-        *reinterpret_cast<uint32_t *>(out_row + (col >> 1)) = pack_e2m1x8(q);
-    }
+    if (FMT == TK_E4M3) st_stream8(out_row + col, pack_e4m3x8<CLAMP>(q));
+    else st_stream4(out_row + (col >> 1), pack_e2m1x8(q));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -201,29 +283,41 @@ __device__ __forceinline__ void sf_store(const SfRef &s, int m, int k, const Sca
     }
 }
 
-// Write the scales of one 16-row tile, staged in LDS as stage[row][g] (fp32 bits or exponent
-// byte), to a column-major layout so that 16 consecutive lanes fill one 64-byte segment.
+// Write the fp32 scales of one tile, staged in LDS as stage[row][g], to the row-major layout:
+// consecutive lanes take consecutive groups of a row, so each row leaves as one contiguous run.
+template <int ROWS, int GPR>
+__device__ __forceinline__ void sf_store_tile_rowmajor(const SfRef &s, const uint32_t (*stage)[GPR], int m0, int k0) {
+    for (int e = threadIdx.x; e < ROWS * GPR; e += kThreads) {
+        const int r = e / GPR, g = e % GPR;
+        const int m = m0 + r, k = k0 + g;
+        if (m < s.nm && k < s.nk) st_stream4(reinterpret_cast<uint32_t *>(s.base) + (int64_t)m * s.ld + k, stage[r][g]);
+    }
+}
+
+// Write the scales of one tile of ROWS rows, staged in LDS as stage[row][g] (fp32 bits or exponent
+// byte), to a column-major layout: consecutive lanes take consecutive rows, so ROWS lanes fill one
+// contiguous 4*ROWS-byte segment.
 //   GPS    : groups per row in the stage
 //   m0, k0 : block coordinates of stage[0][0]
-template <int GPS>
+template <int ROWS, int GPS>
 __device__ __forceinline__ void sf_store_tile_colmajor(const SfRef &s, const uint32_t (*stage)[GPS], int m0, int k0) {
     if (s.layout == TK_SF_COL_F32) {
-        for (int e = threadIdx.x; e < GPS * kTileRows; e += kThreads) {
-            const int g = e / kTileRows, r = e % kTileRows;
+        for (int e = threadIdx.x; e < GPS * ROWS; e += kThreads) {
+            const int g = e / ROWS, r = e % ROWS;
             const int m = m0 + r, k = k0 + g;
-            if (m < s.nm && k < s.nk) reinterpret_cast<uint32_t *>(s.base)[(int64_t)k * s.ld + m] = stage[r][g];
+            if (m < s.nm && k < s.nk) st_stream4(reinterpret_cast<uint32_t *>(s.base) + (int64_t)k * s.ld + m, stage[r][g]);
         }
     } else {
         constexpr int WPS = (GPS + 3) / 4;   // words per row in the stage
-        for (int e = threadIdx.x; e < WPS * kTileRows; e += kThreads) {
-            const int wd = e / kTileRows, r = e % kTileRows;
+        for (int e = threadIdx.x; e < WPS * ROWS; e += kThreads) {
+            const int wd = e / ROWS, r = e % ROWS;
             const int m = m0 + r, k = k0 + 4 * wd;
             if (m < s.nm && k < s.nk) {
                 uint32_t word = 0;
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                     if (4 * wd + j < GPS && k + j < s.nk) word |= (stage[r][4 * wd + j] & 0xFFu) << (8 * j);
-                *reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(s.base) + (int64_t)(k >> 2) * s.ld + 4 * (int64_t)m) = word;
+                st_stream4(reinterpret_cast<uint8_t *>(s.base) + (int64_t)(k >> 2) * s.ld + 4 * (int64_t)m, word);
             }
         }
     }
