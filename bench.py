@@ -114,26 +114,41 @@ class Workload:
 
 
 def time_gpu(w: Workload, steps: int, warmup: int):
-    """Returns (wall seconds for `steps` launches, list of per-launch kernel durations in us)."""
+    """Returns (wall seconds for `steps` launches, HIP-event microseconds per launch over the same
+    timed region, list of single-launch durations from per-launch event pairs)."""
     for i in range(warmup):
         w.launch(i)
     torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    e0.record()          # torch's current stream is the stream the launches go to
     for i in range(steps):
         w.launch(i)
+    e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    # per-launch kernel duration: one HIP event pair around each launch, on the launch stream
+    region_us = e0.elapsed_time(e1) * 1e3 / steps
+    # single launches: one event pair around each (adds the cost of the two event records)
     n = min(steps, 200)
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
-    torch.cuda.synchronize()
     for i in range(n):
         ev[i][0].record()
         w.launch(i)
         ev[i][1].record()
     torch.cuda.synchronize()
     per = [a.elapsed_time(b) * 1e3 for a, b in ev]
-    return wall, per
+    return wall, region_us, per
+
+
+def copy_calibration(n_copies: int = 20, mib: int = 256):
+    """Plain device copies of a known size, so that a hardware-counter run of this script also
+    holds a kernel whose HBM bytes are known (reads `mib` MiB, writes `mib` MiB per copy)."""
+    src = torch.arange((mib << 20) // 4, dtype=torch.int32, device='cuda:0')
+    dst = torch.empty_like(src)
+    for _ in range(n_copies):
+        torch.add(src, 1, out=dst)      # an ordinary elementwise kernel: one read and one write per element
+    torch.cuda.synchronize()
+    return {'copy_calibration': {'copies': n_copies, 'bytes_read_each': mib << 20, 'bytes_written_each': mib << 20}}
 
 
 def cpu_baseline(w: Workload, budget_s: float = 12.0):
@@ -185,8 +200,7 @@ def cpu_baseline(w: Workload, budget_s: float = 12.0):
 
 def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool):
     w = Workload(cfg)
-    wall, per = time_gpu(w, steps, warmup)
-    kern_us = statistics.mean(per)
+    wall, kern_us, per = time_gpu(w, steps, warmup)
     ms_per_step = wall / steps * 1e3
     value = w.bytes / (wall / steps) / 1e9
     achieved = w.bytes / (kern_us * 1e-6) / 1e9
@@ -200,8 +214,8 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool):
         'us_per_call': round(ms_per_step * 1e3, 3), 'pct_of_hbm_peak': round(100 * value / HBM_PEAK_GBS, 2),
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
                      'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': None,
-                     'kernel_us_mean': round(kern_us, 3), 'kernel_us_median': round(statistics.median(per), 3),
-                     'kernel_us_min': round(min(per), 3)},
+                     'kernel_us': round(kern_us, 3), 'timing': f'HIP events around the {steps} timed launches / {steps}',
+                     'single_launch_us_median': round(statistics.median(per), 3), 'single_launch_us_min': round(min(per), 3)},
     }
     if with_cpu:
         line['cpu_baseline'], line['parity'] = cpu_baseline(w)
@@ -211,11 +225,14 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=2000)
-    ap.add_argument('--warmup', type=int, default=200)
+    ap.add_argument('--steps', type=int, default=5000)
+    ap.add_argument('--warmup', type=int, default=2000,
+                    help='untimed launches first; the GPU needs ~15 ms of load to reach its steady clocks')
     ap.add_argument('--config', type=int, default=3, choices=sorted(WORKLOADS))
     ap.add_argument('--all-configs', action='store_true', help='also print one line per other configuration to stderr')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU-oracle baseline / parity leg')
+    ap.add_argument('--copy-calibration', action='store_true',
+                    help='also run plain device copies of known size (reference kernel for hardware-counter runs)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: this path has no multi-GPU component (rows are independent; '
@@ -226,7 +243,10 @@ def main():
         for cfg in sorted(WORKLOADS):
             if cfg != args.config:
                 print(json.dumps(bench_config(cfg, args.steps, args.warmup, not args.no_cpu)), file=sys.stderr, flush=True)
-    print(json.dumps(bench_config(args.config, args.steps, args.warmup, not args.no_cpu)), flush=True)
+    line = bench_config(args.config, args.steps, args.warmup, not args.no_cpu)
+    if args.copy_calibration:
+        line.update(copy_calibration())
+    print(json.dumps(line), flush=True)
 
 
 if __name__ == '__main__':

@@ -1,0 +1,172 @@
+"""C-ABI checks that need no GPU: the library loads, exports every symbol the header declares, and
+its host-side validation returns the documented status codes (no kernel is ever launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, 'include', 'tk_quant.h')
+
+
+@pytest.fixture(scope='module')
+def lib():
+    from tilekernels_amd import _ffi
+    return _ffi.load()
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(tk_[a-z_0-9]+)\s*\(', text)))
+
+
+def test_header_symbols_are_exported_and_bound(lib):
+    from tilekernels_amd import _ffi
+    names = declared_symbols()
+    assert len(names) >= 8
+    for n in names:
+        assert hasattr(lib, n), f'{n} declared in tk_quant.h but not exported'
+        assert n in _ffi.SIGNATURES, f'{n} has no ctypes signature'
+    assert sorted(_ffi.SIGNATURES) == names
+
+
+def test_version_and_strerror(lib):
+    text = open(HEADER).read()
+    want = int(re.search(r'#define TK_QUANT_VERSION (\d+)', text).group(1))
+    assert lib.tk_version() == want
+    assert lib.tk_strerror(0) == b'ok'
+    for code in range(-11, 0):
+        assert lib.tk_strerror(code) not in (b'', b'ok', b'unknown status')
+    assert lib.tk_strerror(-99) == b'unknown status'
+    assert lib.tk_strerror(700) == b'hip error'
+
+
+# status codes of enum tk_status
+OK, NULLP, SHAPE, DTYPE, FMT, GROUP, LAYOUT, MODE, STRIDE, ALIGN, LARGE, VALUE = 0, -1, -2, -3, -4, -5, -6, -7, -8, -9, -10, -11
+P = 0x10000   # a fake, well-aligned, non-null device address (never dereferenced by the checks)
+
+
+def check_pt(lib, x=P, dt=0, M=64, K=1024, ld=None, out=P, sf=P, sf_ld=None, fmt=0, group=128, layout=0, rnd=0, mode=0):
+    ld = K if ld is None else ld
+    nk = -(-K // group) if group > 0 else 1
+    if sf_ld is None:
+        sf_ld = nk if layout == 0 else (M + 3) // 4 * 4 if layout == 1 else (4 * M + 15) // 16 * 16
+    return lib.tk_check_per_token_cast(x, dt, M, K, ld, out, sf, sf_ld, fmt, group, layout, rnd, mode)
+
+
+def test_per_token_cast_validation(lib):
+    assert check_pt(lib) == OK
+    assert check_pt(lib, M=0, x=0, out=0, sf=0) == OK                  # empty input: nothing to check
+    assert check_pt(lib, dt=2) == DTYPE
+    assert check_pt(lib, fmt=2) == FMT
+    assert check_pt(lib, mode=3) == MODE
+    assert check_pt(lib, layout=3) == LAYOUT
+    assert check_pt(lib, layout=2, rnd=0) == LAYOUT                    # UE8M0 bytes need power-of-two scales
+    assert check_pt(lib, layout=2, rnd=1) == OK
+    assert check_pt(lib, K=1020) == SHAPE
+    assert check_pt(lib, M=-1) == SHAPE
+    assert check_pt(lib, group=48) == GROUP
+    assert check_pt(lib, K=1024, group=1024) == OK                     # one scale per row
+    assert check_pt(lib, K=1000, group=1000) == GROUP                  # ... needs K % 64 == 0
+    assert check_pt(lib, K=1024, group=1024, mode=1) == MODE
+    assert check_pt(lib, x=0) == NULLP
+    assert check_pt(lib, out=0) == NULLP
+    assert check_pt(lib, out=0, mode=1) == OK                          # sf-only needs no output
+    assert check_pt(lib, sf=0) == NULLP
+    assert check_pt(lib, ld=512) == STRIDE
+    assert check_pt(lib, sf_ld=4) == STRIDE
+    assert check_pt(lib, x=P + 2) == ALIGN
+    assert check_pt(lib, ld=1028) == ALIGN
+    assert check_pt(lib, out=P + 4) == ALIGN
+    assert check_pt(lib, M=2 ** 31) == LARGE
+
+
+def check_pb(lib, x=P, dt=0, M=256, K=512, out=P, sf=P, sf_ld=None, fmt=0, bm=128, bk=128, layout=0, rnd=0, mode=0):
+    if sf_ld is None:
+        nm, nk = -(-M // bm), -(-K // bk)
+        sf_ld = nk if layout == 0 else (nm + 3) // 4 * 4 if layout == 1 else (4 * nm + 15) // 16 * 16
+    return lib.tk_check_per_block_cast(x, dt, M, K, out, sf, sf_ld, fmt, bm, bk, layout, rnd, mode)
+
+
+def test_per_block_cast_validation(lib):
+    assert check_pb(lib) == OK
+    for bm, bk in ((32, 32), (32, 128), (128, 32)):
+        assert check_pb(lib, bm=bm, bk=bk) == OK
+    assert check_pb(lib, bm=64) == GROUP
+    assert check_pb(lib, bk=1) == GROUP
+    assert check_pb(lib, K=96) == SHAPE                                 # K % 64
+    assert check_pb(lib, mode=2, layout=1) == LAYOUT                    # given scales are row-major only
+    assert check_pb(lib, layout=2, rnd=0) == LAYOUT
+    assert check_pb(lib, x=P + 8) == ALIGN
+    assert check_pb(lib, sf=0) == NULLP
+    assert check_pb(lib, sf_ld=1) == STRIDE
+    assert check_pb(lib, M=0, x=0, out=0, sf=0) == OK
+    assert check_pb(lib, dt=7) == DTYPE
+
+
+def check_sw(lib, x=P, dt=0, R=64, H=2048, out=P, sf=P, sf_ld=None, group=128, layout=0, rnd=0, floor=-1.0,
+             ptt=0, w=0, nw=0, pe=0, use_clamp=0, clamp=0.0, cnt=0):
+    if sf_ld is None:
+        nk = H // group if group else 1
+        sf_ld = nk if layout == 0 else (R + 3) // 4 * 4 if layout == 1 else (4 * R + 15) // 16 * 16
+    return lib.tk_check_swiglu_per_token_cast(x, dt, R, H, out, sf, sf_ld, group, layout, rnd, floor, ptt, w, nw, pe,
+                                              use_clamp, clamp, cnt)
+
+
+def test_swiglu_validation(lib):
+    assert check_sw(lib) == OK
+    assert check_sw(lib, group=2048) == OK
+    assert check_sw(lib, group=2048, layout=1) == LAYOUT                # one scale per row: row-major only
+    assert check_sw(lib, group=256) == GROUP
+    assert check_sw(lib, H=2000) == SHAPE
+    assert check_sw(lib, R=-5) == SHAPE
+    assert check_sw(lib, cnt=P) == MODE                                 # counters need a clamp
+    assert check_sw(lib, cnt=P, use_clamp=1, clamp=1.0) == OK
+    assert check_sw(lib, cnt=P + 4, use_clamp=1, clamp=1.0) == ALIGN
+    assert check_sw(lib, use_clamp=1, clamp=float('nan')) == VALUE
+    assert check_sw(lib, floor=float('nan')) == VALUE
+    assert check_sw(lib, ptt=P) == NULLP                                # index without weights
+    assert check_sw(lib, ptt=P, w=P, nw=128) == OK
+    assert check_sw(lib, layout=2, rnd=0) == LAYOUT
+    assert check_sw(lib, layout=2, rnd=1) == OK
+    assert check_sw(lib, x=P + 4) == ALIGN
+    assert check_sw(lib, out=0) == NULLP
+    assert check_sw(lib, R=0, x=0, out=0, sf=0) == OK
+    assert check_sw(lib, sf_ld=3) == STRIDE
+
+
+def test_launching_entry_points_reject_before_touching_the_device(lib):
+    """A rejected call returns the status from the same validation and launches nothing, so it is safe
+    without a GPU."""
+    assert lib.tk_per_token_cast(P, 0, 64, 1020, 1020, P, P, 8, 0, 128, 0, 0, 0, None) == SHAPE
+    assert lib.tk_per_block_cast(P, 0, 64, 512, P, P, 4, 0, 64, 64, 0, 0, 0, None) == GROUP
+    assert lib.tk_swiglu_per_token_cast(P, 0, 64, 2000, P, P, 16, 128, 0, 0, -1.0, None, None, 0, None, 0, 0.0, None, 0, None) == SHAPE
+    assert lib.tk_per_token_cast(None, 0, 0, 1024, 1024, None, None, 8, 0, 128, 0, 0, 0, None) == OK     # M == 0
+
+
+def test_host_side_geometry_matches_the_oracle_layouts():
+    """Scale-tensor shapes/strides produced by the host wrapper (allocation + epilogue) equal the oracle's."""
+    import torch
+    from oracle import torch_ref
+    from tilekernels_amd.quant.common import alloc_scaling_factors, cast_epilogue, get_cast_output_config, sf_leading_dim
+    for (M, K, blk) in ((37, 576, (1, 128)), (4001, 7168, (1, 32)), (130, 2560, (128, 128)), (1, 64, (1, 64)), (5, 512, (32, 32))):
+        x = torch.zeros((M, K), dtype=torch.bfloat16)
+        for col, rnd, packed in ((False, False, False), (True, False, False), (True, True, True)):
+            cfg = get_cast_output_config('e4m3', blk, col, rnd, packed)
+            store = alloc_scaling_factors((M, K), cfg, 'cpu')
+            got = cast_epilogue(store, M, K, cfg)
+            _, want = torch_ref.cast(x, 'e4m3', blk, round_sf=rnd, use_tma_aligned_col_major_sf=col, use_packed_ue8m0=packed)
+            assert got.dtype == want.dtype and got.shape == want.shape and got.stride() == want.stride(), (M, K, blk, col, packed)
+            nm, nk = -(-M // blk[0]), -(-K // blk[1])
+            need = nk if not col else (4 * nm if packed else nm)
+            assert sf_leading_dim(store) >= need
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from tilekernels_amd import _ffi
+    monkeypatch.setattr(_ffi, '_lib', None)
+    monkeypatch.setattr(_ffi, 'LIB_PATH', str(tmp_path / 'nope.so'))
+    with pytest.raises(ImportError):
+        _ffi.load()

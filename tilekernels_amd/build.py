@@ -24,6 +24,8 @@ FLAGS = [
     '-fno-gpu-flush-denormals-to-zero',
     # keep packed-fp32 VALU instructions out of the generated code
     '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+    # the first 16 dwords of kernel arguments arrive preloaded in SGPRs at wave start
+    '-mllvm', '-amdgpu-kernarg-preload-count=16',
     '-Wall', '-Wno-unused-command-line-argument',
 ]
 

@@ -11,8 +11,6 @@
 //
 // Reference semantics: tile_kernels/quant/per_token_cast_kernel.py:65-154 (plain-tensor branch),
 // tile_kernels/quant/common.py:196-244.
-#include <stdlib.h>
-
 #include "tk_device.hpp"
 #include "tk_host.hpp"
 
@@ -28,24 +26,36 @@ struct PerTokenParams {
     int round_sf, mode;
 };
 
+// Parameters travel as individual scalars (16 dwords in all) so that they are preloaded into SGPRs
+// at wave start (the library is built with -amdgpu-kernarg-preload-count=16).
+#define TK_PT_KERNEL_ARGS                                                                                 \
+    const void *a_x, uint8_t *a_out, void *a_sf, int64_t a_sf_ld, int64_t a_x_ld, int a_M, int a_K, int a_tiles_k, \
+        int a_round_sf, int a_mode, int a_sf_layout, int a_nk
+#define TK_PT_KERNEL_UNPACK \
+    const PerTokenParams p{a_x, a_out, SfRef{a_sf, a_sf_ld, a_sf_layout, a_M, a_nk}, a_x_ld, a_M, a_K, a_tiles_k, a_round_sf, a_mode}
+#define TK_PT_LAUNCH_ARGS(p) \
+    (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).x_ld, (p).M, (p).K, (p).tiles_k, (p).round_sf, (p).mode, (p).sf.layout, (p).sf.nk
+
 // Tile shapes (RPW = rows per wave):
-//   WIDE  (row-major scales):      RPW rows x 2048 columns, the 4 waves side by side on the same rows;
+//   WIDE  (row-major scales):      RPW rows x (W*512) columns, W = blockDim.x/64 waves side by side on the same rows;
 //         the tile's scales are RPW contiguous runs, staged in LDS and stored as whole segments
 //   !WIDE (column-major layouts):  4*RPW rows x 512 columns, the 4 waves stacked; the staged scales
 //         are stored transposed, 4*RPW rows per contiguous segment
 // FULL: the tile grid covers the matrix exactly, so no bounds checks are compiled in.
 template <typename InT, int G, int FMT, int RPW, bool WIDE, bool FULL>
-__global__ __launch_bounds__(kThreads) void per_token_cast_kernel(const PerTokenParams p) {
+__global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_token_cast_kernel(TK_PT_KERNEL_ARGS) {
+    TK_PT_KERNEL_UNPACK;
     constexpr int LPG = G / 8;            // lanes per group
     constexpr int GPS = kStripCols / G;   // groups per 512-column strip
     constexpr int ROWS = WIDE ? RPW : kWaves * RPW;       // rows per tile
-    constexpr int SGPR = WIDE ? kWaves * GPS : GPS;       // staged groups per row
+    constexpr int SGPR = WIDE ? kMaxWideWaves * GPS : GPS;   // staged groups per row (capacity)
+    const int nwaves = WIDE ? (int)(blockDim.x >> 6) : kWaves;
     using RS = RowScales<Fmt<FMT>::qmax, RPW, LPG>;
     __shared__ uint32_t stage[ROWS][SGPR];
 
     const int tile_m = blockIdx.x / p.tiles_k, tile_k = blockIdx.x - tile_m * p.tiles_k;
     const int lane = threadIdx.x & 63, wave = wave_id();
-    const int strip = WIDE ? tile_k * kWaves + wave : tile_k;
+    const int strip = WIDE ? tile_k * nwaves + wave : tile_k;
     const int col = strip * kStripCols + lane * 8;
     const int g_in_strip = lane / LPG;
     const int kgrp = strip * GPS + g_in_strip;
@@ -104,7 +114,7 @@ __global__ __launch_bounds__(kThreads) void per_token_cast_kernel(const PerToken
     }
     if (p.mode != TK_CAST_GIVEN_SF) {
         __syncthreads();
-        if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
+        if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
         else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
     }
 }
@@ -113,7 +123,8 @@ __global__ __launch_bounds__(kThreads) void per_token_cast_kernel(const PerToken
 // served by L2).  Reference: the `hidden == num_per_channels` branch,
 // tile_kernels/quant/per_token_cast_kernel.py:31-35.
 template <typename InT, int FMT>
-__global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(const PerTokenParams p) {
+__global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERNEL_ARGS) {
+    TK_PT_KERNEL_UNPACK;
     __shared__ uint32_t part[kThreads / 16];
     const int row = blockIdx.x;
     const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row * p.x_ld;
@@ -144,27 +155,23 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(const PerT
     }
 }
 
-// rows per wave; 1, 2 or 4 (TK_PT_RPW overrides the default for tuning runs)
-static int per_token_rpw() {
-    static const int v = [] {
-        const char *e = getenv("TK_PT_RPW");
-        const int r = e ? atoi(e) : 2;
-        return (r == 1 || r == 2 || r == 4) ? r : 2;
-    }();
-    return v;
-}
+// Rows per wave.  Measured on MI355X (us per call): bf16 [4096, 7168] -> E4M3 1x128 row-major scales
+// 18.1 / 16.3 / 17.0 for 1 / 2 / 4 rows; bf16 [16384, 7168] -> E2M1 1x32 packed scales 55.2 / 43.4 / 45.4.
+constexpr int kPerTokenRowsPerWave = 2;
 
 template <typename InT, int G, int FMT, int RPW, bool WIDE>
 static void launch_per_token_4(PerTokenParams &p, hipStream_t stream) {
-    constexpr int ROWS = WIDE ? RPW : kWaves * RPW;
-    constexpr int COLS = WIDE ? kWaves * kStripCols : kStripCols;
-    const int tiles_m = (p.M + ROWS - 1) / ROWS;
-    p.tiles_k = (p.K + COLS - 1) / COLS;
-    const dim3 grid((unsigned)(tiles_m * p.tiles_k)), block(kThreads);
-    if (p.M % ROWS == 0 && p.K % COLS == 0)
-        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, true>), grid, block, 0, stream, p);
+    const int strips = (p.K + kStripCols - 1) / kStripCols;
+    const int waves = WIDE ? wide_tile_waves(strips) : kWaves;
+    const int rows = WIDE ? RPW : kWaves * RPW;
+    const int cols = WIDE ? waves * kStripCols : kStripCols;
+    const int tiles_m = (p.M + rows - 1) / rows;
+    p.tiles_k = (p.K + cols - 1) / cols;
+    const dim3 grid((unsigned)(tiles_m * p.tiles_k)), block(64 * waves);
+    if (p.M % rows == 0 && p.K % cols == 0)
+        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, true>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
     else
-        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, false>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, false>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
 }
 
 template <typename InT, int G, int FMT, int RPW>
@@ -176,17 +183,13 @@ static void launch_per_token_3(PerTokenParams &p, hipStream_t stream) {
 
 template <typename InT, int G, int FMT>
 static void launch_per_token_2(PerTokenParams &p, hipStream_t stream) {
-    switch (per_token_rpw()) {
-        case 1: launch_per_token_3<InT, G, FMT, 1>(p, stream); break;
-        case 4: launch_per_token_3<InT, G, FMT, 4>(p, stream); break;
-        default: launch_per_token_3<InT, G, FMT, 2>(p, stream); break;
-    }
+    launch_per_token_3<InT, G, FMT, kPerTokenRowsPerWave>(p, stream);
 }
 
 template <typename InT, int FMT>
 static hipError_t launch_per_token(PerTokenParams &p, int group, hipStream_t stream) {
     if (group == p.K && group != 16 && group != 32 && group != 64 && group != 128) {
-        hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT>), dim3(p.M), dim3(kThreads), 0, stream, p);
+        hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT>), dim3(p.M), dim3(kThreads), 0, stream, TK_PT_LAUNCH_ARGS(p));
         return hipGetLastError();
     }
     switch (group) {

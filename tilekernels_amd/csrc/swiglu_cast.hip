@@ -9,8 +9,6 @@
 //
 // Reference semantics: tile_kernels/quant/swiglu_forward_and_per_token_cast_kernel.py:61-170,
 // tile_kernels/torch/swiglu.py:62-86.
-#include <stdlib.h>
-
 #include "tk_device.hpp"
 #include "tk_host.hpp"
 
@@ -31,6 +29,21 @@ struct SwigluParams {
     float floor_;        // amax lower clamp
     float clamp;
 };
+
+// The kernels take their parameters as individual scalars, hottest first: the first 16 dwords of the
+// kernel-argument segment are preloaded into SGPRs when a wave starts (the library is built with
+// -amdgpu-kernarg-preload-count=16), which takes a scalar-cache miss off the front of every wave.
+#define TK_SWIGLU_KERNEL_ARGS                                                                                      \
+    const void *a_x, uint8_t *a_out, void *a_sf, int64_t a_sf_ld, int a_R, int a_H, int a_tiles_m, int a_tiles_k, \
+        float a_floor, float a_clamp, int a_round_sf, int a_sf_layout, const int32_t *a_pe, const int32_t *a_ptt, \
+        const float *a_w, unsigned long long *a_cnt, int64_t a_nw, int a_nk
+#define TK_SWIGLU_KERNEL_UNPACK                                                                            \
+    const SwigluParams p{a_x, a_out, SfRef{a_sf, a_sf_ld, a_sf_layout, a_R, a_nk}, a_ptt, a_w, a_pe, a_cnt, \
+                         a_nw, a_R, a_H, a_tiles_m, a_tiles_k, a_round_sf, a_floor, a_clamp}
+#define TK_SWIGLU_LAUNCH_ARGS(p)                                                                                  \
+    (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).R, (p).H, (p).tiles_m, (p).tiles_k, (p).floor_, (p).clamp,       \
+        (p).round_sf, (p).sf.layout, (p).pos_to_expert, (p).pos_to_token_topk, (p).topk_weights, (p).clamped_count, \
+        (p).num_weights, (p).sf.nk
 
 // silu(g) * u = g / (1 + exp(-g)) * u in fp32, built on v_exp_f32 / v_rcp_f32 (about 1 ulp each).
 // The reference's CPU evaluation (vectorised exp, IEEE division) is itself only faithful to about
@@ -113,16 +126,18 @@ __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
 }
 
 // Tile shapes as in the per-token cast (RPW = rows per wave):
-//   WIDE  (row-major scales):     RPW rows x 2048 output columns, the 4 waves side by side; the tile's
+//   WIDE  (row-major scales):     RPW rows x (W*512) output columns, W = blockDim.x/64 waves side by side; the tile's
 //         scales are RPW contiguous runs of 16, staged in LDS and stored as whole segments
 //   !WIDE (column-major layouts): 4*RPW rows x 512 columns, the 4 waves stacked, scales stored transposed
 // FULL: the tile grid covers the matrix exactly: no bounds checks are compiled in.
 // MASK: pos_to_expert is given.
 template <typename InT, int CLAMP, int RPW, bool WIDE, bool FULL, bool MASK>
-__global__ __launch_bounds__(kThreads) void swiglu_cast_kernel(const SwigluParams p) {
+__global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
+    TK_SWIGLU_KERNEL_UNPACK;
     constexpr int GPS = kStripCols / 128;   // 4 groups per strip
     constexpr int ROWS = WIDE ? RPW : kWaves * RPW;
-    constexpr int SGPR = WIDE ? kWaves * GPS : GPS;
+    constexpr int SGPR = WIDE ? kMaxWideWaves * GPS : GPS;   // staged groups per row (capacity)
+    const int nwaves = WIDE ? (int)(blockDim.x >> 6) : kWaves;
     using RS = RowScales<448, RPW, 16>;
     __shared__ uint32_t stage[ROWS][SGPR];
 
@@ -135,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_cast_kernel(const SwigluParam
 
     for (int tile = blockIdx.x; tile < total; tile += gridDim.x) {
         const int tile_m = tile / p.tiles_k, tile_k = tile - tile_m * p.tiles_k;
-        const int strip = WIDE ? tile_k * kWaves + wave : tile_k;
+        const int strip = WIDE ? tile_k * nwaves + wave : tile_k;
         const int col = strip * kStripCols + lane * 8;
         const bool col_ok = FULL || col < p.H;
         const int row0 = tile_m * ROWS + srow;
@@ -206,7 +221,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_cast_kernel(const SwigluParam
             if (col_ok && (FULL || row0 + r < p.R))
                 quantise_store8<TK_E4M3, false>(v[r], rs.inv[r], p.out + (int64_t)(row0 + r) * p.H, col);
         __syncthreads();
-        if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
+        if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
         else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
         if (gridDim.x < total) __syncthreads();   // stage is reused by the next tile
     }
@@ -216,7 +231,8 @@ __global__ __launch_bounds__(kThreads) void swiglu_cast_kernel(const SwigluParam
 // One scale per row (group == H): a workgroup per row, the activation is evaluated twice (amax
 // pass, then convert pass; the second read comes from L2).  Row-major scales only.
 template <typename InT, int CLAMP>
-__global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(const SwigluParams p) {
+__global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KERNEL_ARGS) {
+    TK_SWIGLU_KERNEL_UNPACK;
     __shared__ uint32_t part[kThreads / 16];
     const InT *xb = reinterpret_cast<const InT *>(p.x);
     ClampCounter<CLAMP> counter;
@@ -267,31 +283,27 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(const SwigluP
     counter.flush(p.clamped_count);
 }
 
-// rows per wave of the tiled kernel; 1, 2 or 4 (TK_SWIGLU_RPW overrides the default for tuning runs)
-static int swiglu_rpw() {
-    static const int v = [] {
-        const char *e = getenv("TK_SWIGLU_RPW");
-        const int r = e ? atoi(e) : 2;
-        return (r == 1 || r == 2 || r == 4) ? r : 2;
-    }();
-    return v;
-}
+// Rows per wave of the tiled kernel.  Measured on MI355X at [8192, 4096] bf16 (us per call, row-major
+// scales): 1 row 16.5, 2 rows 15.7, 4 rows 15.0.
+constexpr int kSwigluRowsPerWave = 4;
 
 template <typename InT, int CLAMP, int RPW, bool WIDE>
 static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t stream) {
-    constexpr int ROWS = WIDE ? RPW : kWaves * RPW;
-    constexpr int COLS = WIDE ? kWaves * kStripCols : kStripCols;
-    p.tiles_m = (p.R + ROWS - 1) / ROWS;
-    p.tiles_k = (p.H + COLS - 1) / COLS;
+    const int strips = (p.H + kStripCols - 1) / kStripCols;
+    const int waves = WIDE ? wide_tile_waves(strips) : kWaves;
+    const int rows = WIDE ? RPW : kWaves * RPW;
+    const int cols = WIDE ? waves * kStripCols : kStripCols;
+    p.tiles_m = (p.R + rows - 1) / rows;
+    p.tiles_k = (p.H + cols - 1) / cols;
     const int total = p.tiles_m * p.tiles_k;
-    const dim3 grid((unsigned)((max_blocks > 0 && max_blocks < total) ? max_blocks : total)), block(kThreads);
-    const bool full = p.R % ROWS == 0 && p.H % COLS == 0;
+    const dim3 grid((unsigned)((max_blocks > 0 && max_blocks < total) ? max_blocks : total)), block(64 * waves);
+    const bool full = p.R % rows == 0 && p.H % cols == 0;
     if (p.pos_to_expert) {
-        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, true, true>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, false, true>), grid, block, 0, stream, p);
+        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, true, true>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, false, true>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
     } else {
-        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, true, false>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, false, false>), grid, block, 0, stream, p);
+        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, true, false>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, false, false>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
     }
 }
 
@@ -299,22 +311,10 @@ template <typename InT, int CLAMP>
 static hipError_t launch_swiglu_2(SwigluParams &p, bool row_group, int max_blocks, hipStream_t stream) {
     if (row_group) {
         const int grid = max_blocks > 0 && max_blocks < p.R ? max_blocks : p.R;
-        hipLaunchKernelGGL((swiglu_rowgroup_kernel<InT, CLAMP>), dim3(grid), dim3(kThreads), 0, stream, p);
+        hipLaunchKernelGGL((swiglu_rowgroup_kernel<InT, CLAMP>), dim3(grid), dim3(kThreads), 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
     } else {
-        const int rpw = swiglu_rpw();
-        if (p.sf.layout == TK_SF_ROW_F32) {
-            switch (rpw) {
-                case 1: launch_swiglu_tiled<InT, CLAMP, 1, true>(p, max_blocks, stream); break;
-                case 4: launch_swiglu_tiled<InT, CLAMP, 4, true>(p, max_blocks, stream); break;
-                default: launch_swiglu_tiled<InT, CLAMP, 2, true>(p, max_blocks, stream); break;
-            }
-        } else {
-            switch (rpw) {
-                case 1: launch_swiglu_tiled<InT, CLAMP, 1, false>(p, max_blocks, stream); break;
-                case 4: launch_swiglu_tiled<InT, CLAMP, 4, false>(p, max_blocks, stream); break;
-                default: launch_swiglu_tiled<InT, CLAMP, 2, false>(p, max_blocks, stream); break;
-            }
-        }
+        if (p.sf.layout == TK_SF_ROW_F32) launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, true>(p, max_blocks, stream);
+        else launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, false>(p, max_blocks, stream);
     }
     return hipGetLastError();
 }

@@ -11,8 +11,17 @@
 namespace tk {
 
 constexpr int kStripCols = 512;   // columns one wave covers per row: 64 lanes x 8 elements
-constexpr int kThreads = 256;     // 4 waves per workgroup
+constexpr int kThreads = 256;     // 4 waves per workgroup (stacked tiles; wide tiles use 3..8 waves)
 constexpr int kWaves = kThreads / 64;
+constexpr int kMaxWideWaves = 8;
+
+// Number of waves of a wide tile (waves side by side, 512 columns each) for a row of `strips`
+// 512-column strips: the largest of 8..3 that divides it, so that no wave idles; 4 if none does.
+inline int wide_tile_waves(int strips) {
+    for (int w = kMaxWideWaves; w >= 3; --w)
+        if (strips % w == 0) return w;
+    return 4;
+}
 
 struct bf16_t { uint16_t bits; };
 
@@ -283,12 +292,13 @@ __device__ __forceinline__ void sf_store(const SfRef &s, int m, int k, const Sca
     }
 }
 
-// Write the fp32 scales of one tile, staged in LDS as stage[row][g], to the row-major layout:
-// consecutive lanes take consecutive groups of a row, so each row leaves as one contiguous run.
-template <int ROWS, int GPR>
-__device__ __forceinline__ void sf_store_tile_rowmajor(const SfRef &s, const uint32_t (*stage)[GPR], int m0, int k0) {
-    for (int e = threadIdx.x; e < ROWS * GPR; e += kThreads) {
-        const int r = e / GPR, g = e % GPR;
+// Write the fp32 scales of one tile, staged in LDS as stage[row][g] (g < gpr <= PITCH), to the
+// row-major layout: consecutive lanes take consecutive groups of a row, so each row leaves as one
+// contiguous run.
+template <int ROWS, int PITCH>
+__device__ __forceinline__ void sf_store_tile_rowmajor(const SfRef &s, const uint32_t (*stage)[PITCH], int gpr, int m0, int k0) {
+    for (int e = threadIdx.x; e < ROWS * gpr; e += blockDim.x) {
+        const int r = e / gpr, g = e - r * gpr;
         const int m = m0 + r, k = k0 + g;
         if (m < s.nm && k < s.nk) st_stream4(reinterpret_cast<uint32_t *>(s.base) + (int64_t)m * s.ld + k, stage[r][g]);
     }
