@@ -31,6 +31,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 LLC_BYTES = 256 << 20
 
+# HBM bytes per launch from rocprofv3 counter runs of this script (FETCH_SIZE and WRITE_SIZE, each
+# scaled by what the same counter reads for the 256 MiB copy of --copy-calibration); the summaries
+# are kept under profiles/.  None where no counter run was made.
+MEASURED_TRAFFIC_BYTES = {1: 89.17e6, 2: None, 3: 84.50e6, 4: None, 5: 297.30e6}
+
 WORKLOADS = {
     1: 'per_token_cast e4m3 1x128, bf16 [4096,7168]',
     2: 'per_block_cast e4m3 128x128, bf16 [7168,2048]',
@@ -213,7 +218,7 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool):
                    'boundary': 'C ABI (ctypes), preallocated outputs'},
         'us_per_call': round(ms_per_step * 1e3, 3), 'pct_of_hbm_peak': round(100 * value / HBM_PEAK_GBS, 2),
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': None,
+                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': MEASURED_TRAFFIC_BYTES[cfg],
                      'kernel_us': round(kern_us, 3), 'timing': f'HIP events around the {steps} timed launches / {steps}',
                      'single_launch_us_median': round(statistics.median(per), 3), 'single_launch_us_min': round(min(per), 3)},
     }

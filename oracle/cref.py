@@ -35,6 +35,8 @@ def lib():
         L.tkref_swiglu.restype = i32
         L.tkref_e4m3_encode_n.argtypes = [vp, i64, vp]
         L.tkref_e2m1_encode_n.argtypes = [vp, i64, vp]
+        L.tkref_count_div_mismatches.argtypes = [f32, ctypes.c_uint32, ctypes.c_uint32, i32]
+        L.tkref_count_div_mismatches.restype = i64
         _lib = L
     return _lib
 
@@ -97,3 +99,9 @@ def swiglu_forward(x: torch.Tensor, pos_to_token_topk=None, topk_weights=None, s
                             _ptr(clamped_count), _ptr(out))
     assert rc == 0
     return out
+
+
+def count_div_mismatches(c: float, lo_bits: int, hi_bits: int, uncorrected: bool = False) -> int:
+    """Positive floats in [lo_bits, hi_bits) (bit patterns) where a*y + fma(-c, a*y, a)*y != a/c
+    (``uncorrected``: where a*y alone != a/c)."""
+    return int(lib().tkref_count_div_mismatches(c, lo_bits, hi_bits, int(uncorrected)))

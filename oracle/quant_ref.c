@@ -177,3 +177,27 @@ void tkref_e4m3_encode_n(const float *v, int64_t n, uint8_t *out) {
 void tkref_e2m1_encode_n(const float *v, int64_t n, uint8_t *out) {
     for (int64_t i = 0; i < n; ++i) out[i] = tkref_e2m1_encode(v[i]);
 }
+
+/*
+ * Support for the test that pins the GPU's three-instruction division by a constant:
+ *   q = a * y;  q' = fma(fma(-c, q, a), y, q)   with y = fl(1 / c)
+ * Counts the positive floats with bit patterns in [lo_bits, hi_bits) for which q' differs from the
+ * IEEE quotient a / c (only inputs whose quotient is a normal number are counted: smaller operands
+ * take an ordinary division on the GPU).  fmaf() is the correctly rounded libm/hardware fma.
+ * `uncorrected` != 0 drops the fma step (q alone), which is NOT exact: the negative control.
+ */
+int64_t tkref_count_div_mismatches(float c, uint32_t lo_bits, uint32_t hi_bits, int uncorrected) {
+    const float y = 1.0f / c;
+    int64_t bad = 0;
+#pragma omp parallel for schedule(static) reduction(+ : bad)
+    for (int64_t b = lo_bits; b < (int64_t)hi_bits; ++b) {
+        const float a = u2f((uint32_t)b);
+        const float want = a / c;
+        if (want < 0x1p-126f) continue;
+        const float q = a * y;
+        const float r = fmaf(-c, q, a);
+        const float q2 = uncorrected ? q : fmaf(r, y, q);
+        bad += q2 != want;
+    }
+    return bad;
+}
