@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define TK_QUANT_VERSION 100 /* major*10000 + minor*100 + patch */
+#define TK_QUANT_VERSION 101 /* major*10000 + minor*100 + patch */
 
 enum tk_dtype { TK_BF16 = 0, TK_F32 = 1 };
 enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1 };
@@ -82,6 +82,25 @@ int tk_per_token_cast(const void *x, int x_dtype, int64_t M, int64_t K, int64_t 
 int tk_check_per_token_cast(const void *x, int x_dtype, int64_t M, int64_t K, int64_t x_row_stride,
                             const void *out, const void *sf, int64_t sf_ld, int fmt, int group, int sf_layout,
                             int round_sf, int mode);
+
+/*
+ * Per-token cast of an input that is itself quantised: x holds E4M3 bytes [M, K] or packed E2M1
+ * bytes [M, K/2] (K, x_row_stride in logical elements) with one dequantisation scale per
+ * x_bm x x_bk block in x_sf (any of the three layouts; UE8M0 bytes decode to 2^(e-127)).
+ * Every element is first dequantised, value = code * scale (one fp32 rounding), then cast as above.
+ * Stands behind tile_kernels.quant.per_token_cast(x=(data, sf), x_block_size=...) 
+ * (tile_kernels/quant/per_token_cast_kernel.py:87-126, tile_kernels/quant/common.py:62-88; oracle
+ * tile_kernels/torch/cast.py:87-99).  Cast-and-scale mode only, group in {16, 32, 64, 128}.
+ *   requirements K % 8 == 0, x_row_stride % 8 == 0, x_bk % 8 == 0; x 8-byte (E4M3) / 4-byte (E2M1) aligned
+ */
+int tk_per_token_cast_quantized(const void *x, int x_fmt, int64_t M, int64_t K, int64_t x_row_stride,
+                                const void *x_sf, int64_t x_sf_ld, int x_sf_layout, int x_bm, int x_bk, void *out,
+                                void *sf, int64_t sf_ld, int fmt, int group, int sf_layout, int round_sf,
+                                void *stream);
+int tk_check_per_token_cast_quantized(const void *x, int x_fmt, int64_t M, int64_t K, int64_t x_row_stride,
+                                      const void *x_sf, int64_t x_sf_ld, int x_sf_layout, int x_bm, int x_bk,
+                                      const void *out, const void *sf, int64_t sf_ld, int fmt, int group,
+                                      int sf_layout, int round_sf);
 
 /*
  * Per-block cast: x[M, K] contiguous is cut into bm x bk blocks (bm, bk in {32, 128}; edge blocks

@@ -178,3 +178,30 @@ def test_packed_scales_read_back():
     _, f = tk.quant.per_token_cast(x, 'e2m1', 32, round_sf=True)
     by = packed_sf_bytes(pk, 48)
     assert torch.equal((by.to(torch.int32) << 23).view(torch.float32), f.cpu())
+
+
+def _to_gpu_like(t: torch.Tensor) -> torch.Tensor:
+    """Copy to the GPU keeping the strides (column-major scale views are not dense)."""
+    g = torch.empty_strided(t.shape, t.stride(), dtype=t.dtype, device='cuda')
+    g.copy_(t)
+    return g
+
+
+@pytest.mark.parametrize('mode', [(False, True, False), (True, True, True), (True, True, False), (False, False, False)], ids=_mode_id)
+@pytest.mark.parametrize('fmt', ['e4m3', 'e2m1'])
+@pytest.mark.parametrize('in_fmt', ['e4m3', 'e2m1'])
+@pytest.mark.parametrize('x_block', [(128, 128), (32, 32), (1, 128), (1, 32)])
+@pytest.mark.parametrize('M,K,N', [(401, 7168, 128), (401, 7168, 32), (37, 576, 128), (37, 576, 32), (130, 2048, 64)])
+def test_per_token_cast_of_quantised_input(M, K, N, x_block, in_fmt, fmt, mode):
+    """Input = (codes, scales) of an earlier cast, in every scale layout; same structure as the
+    quantised-input cases of the reference's tests/quant/test_per_token_cast.py:25-36."""
+    tk = _tk()
+    col, rnd, packed = mode
+    kw = dict(use_tma_aligned_col_major_sf=col, round_sf=rnd, use_packed_ue8m0=packed)
+    x = torch.randn((M, K)).to(torch.bfloat16)
+    q = torch_ref.cast(x, in_fmt, x_block, **kw)
+    want_codes, want_sf = torch_ref.cast(q, fmt, (1, N), x_block_size=x_block, **kw)
+    qg = (q[0].cuda(), _to_gpu_like(q[1]))
+    codes, sf = tk.quant.per_token_cast(qg, fmt, N, x_block_size=x_block, **kw)
+    assert_same(codes, want_codes, 'codes')
+    assert_same(sf, want_sf, 'sf')

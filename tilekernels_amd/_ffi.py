@@ -21,6 +21,10 @@ _i64, _i32, _vp, _f32 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_
 SIGNATURES = {
     'tk_per_token_cast': (_i32, [_vp, _i32, _i64, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
     'tk_check_per_token_cast': (_i32, [_vp, _i32, _i64, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32]),
+    'tk_per_token_cast_quantized': (_i32, [_vp, _i32, _i64, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _vp, _i64, _i32,
+                                           _i32, _i32, _i32, _vp]),
+    'tk_check_per_token_cast_quantized': (_i32, [_vp, _i32, _i64, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _vp, _i64,
+                                                 _i32, _i32, _i32, _i32]),
     'tk_per_block_cast': (_i32, [_vp, _i32, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
     'tk_check_per_block_cast': (_i32, [_vp, _i32, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _i32]),
     'tk_swiglu_per_token_cast': (_i32, [_vp, _i32, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _f32, _vp, _vp, _i64,

@@ -20,21 +20,26 @@ struct PerTokenParams {
     const void *x;
     uint8_t *out;
     SfRef sf;
-    int64_t x_ld;     // elements between rows of x
+    int64_t x_ld;     // (logical) elements between rows of x
     int M, K;
     int tiles_k;
     int round_sf, mode;
+    SfRef xsf;        // quantised input only: its block scales ...
+    int in_bm, in_bk; // ... and their block shape
 };
 
 // Parameters travel as individual scalars (16 dwords in all) so that they are preloaded into SGPRs
 // at wave start (the library is built with -amdgpu-kernarg-preload-count=16).
 #define TK_PT_KERNEL_ARGS                                                                                 \
     const void *a_x, uint8_t *a_out, void *a_sf, int64_t a_sf_ld, int64_t a_x_ld, int a_M, int a_K, int a_tiles_k, \
-        int a_round_sf, int a_mode, int a_sf_layout, int a_nk
-#define TK_PT_KERNEL_UNPACK \
-    const PerTokenParams p{a_x, a_out, SfRef{a_sf, a_sf_ld, a_sf_layout, a_M, a_nk}, a_x_ld, a_M, a_K, a_tiles_k, a_round_sf, a_mode}
-#define TK_PT_LAUNCH_ARGS(p) \
-    (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).x_ld, (p).M, (p).K, (p).tiles_k, (p).round_sf, (p).mode, (p).sf.layout, (p).sf.nk
+        int a_round_sf, int a_mode, int a_sf_layout, int a_nk, void *a_xsf, int64_t a_xsf_ld, int a_xsf_layout,      \
+        int a_xsf_nm, int a_xsf_nk, int a_in_bm, int a_in_bk
+#define TK_PT_KERNEL_UNPACK                                                                                          \
+    const PerTokenParams p{a_x, a_out, SfRef{a_sf, a_sf_ld, a_sf_layout, a_M, a_nk}, a_x_ld, a_M, a_K, a_tiles_k,   \
+                           a_round_sf, a_mode, SfRef{a_xsf, a_xsf_ld, a_xsf_layout, a_xsf_nm, a_xsf_nk}, a_in_bm, a_in_bk}
+#define TK_PT_LAUNCH_ARGS(p)                                                                                         \
+    (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).x_ld, (p).M, (p).K, (p).tiles_k, (p).round_sf, (p).mode, (p).sf.layout, \
+        (p).sf.nk, (p).xsf.base, (p).xsf.ld, (p).xsf.layout, (p).xsf.nm, (p).xsf.nk, (p).in_bm, (p).in_bk
 
 // Tile shapes (RPW = rows per wave):
 //   WIDE  (row-major scales):      RPW rows x (W*512) columns, W = blockDim.x/64 waves side by side on the same rows;
@@ -63,13 +68,18 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
     const int srow = WIDE ? 0 : wave * RPW;                // first staged row of this wave
     const int row0 = tile_m * ROWS + srow;
     const int64_t out_ld = FMT == TK_E4M3 ? p.K : p.K / 2;
-    const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * p.x_ld + col;
 
     Raw8<InT> raw[RPW];
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
-        if (FULL) raw[r].load(x + (int64_t)r * p.x_ld);
-        else raw[r].load(x + (int64_t)r * p.x_ld, col_ok && row0 + r < p.M);
+        const void *xp = elem_ptr<InT>(p.x, row0 + r, p.x_ld, col);
+        if (FULL) raw[r].load(xp);
+        else raw[r].load(xp, col_ok && row0 + r < p.M);
+        if constexpr (Elem<InT>::quantised) {
+            // the 8 codes of a lane share one input scale (input blocks are at least 32 columns wide)
+            const bool ok = col_ok && (FULL || row0 + r < p.M);
+            raw[r].s = ok ? sf_load(p.xsf, (row0 + r) / p.in_bm, col / p.in_bk) : 0.0f;
+        }
     }
 
     float inv[RPW];
@@ -127,7 +137,7 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERN
     TK_PT_KERNEL_UNPACK;
     __shared__ uint32_t part[kThreads / 16];
     const int row = blockIdx.x;
-    const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row * p.x_ld;
+    const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row * p.x_ld;   // plain (bf16 / fp32) inputs only
     float amax = 0.0f;
     for (int col = threadIdx.x * 8; col < p.K; col += kThreads * 8) {
         Raw8<InT> raw;
@@ -201,6 +211,29 @@ static hipError_t launch_per_token(PerTokenParams &p, int group, hipStream_t str
     return hipGetLastError();
 }
 
+// Quantised input (codes + block scales): the general, bounds-checked kernel only.
+template <typename InT, int FMT>
+static hipError_t launch_per_token_requant(PerTokenParams &p, int group, hipStream_t stream) {
+    const bool wide = p.sf.layout == TK_SF_ROW_F32;
+    const int strips = (p.K + kStripCols - 1) / kStripCols;
+    const int waves = wide ? wide_tile_waves(strips) : kWaves;
+    const int rows = wide ? kPerTokenRowsPerWave : kWaves * kPerTokenRowsPerWave;
+    const int cols = wide ? waves * kStripCols : kStripCols;
+    p.tiles_k = (p.K + cols - 1) / cols;
+    const dim3 grid((unsigned)(((p.M + rows - 1) / rows) * p.tiles_k)), block(64 * waves);
+#define TK_RQ(G)                                                                                                       \
+    if (wide) hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, kPerTokenRowsPerWave, true, false>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p)); \
+    else hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, kPerTokenRowsPerWave, false, false>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p))
+    switch (group) {
+        case 16: TK_RQ(16); break;
+        case 32: TK_RQ(32); break;
+        case 64: TK_RQ(64); break;
+        default: TK_RQ(128); break;
+    }
+#undef TK_RQ
+    return hipGetLastError();
+}
+
 }  // namespace tk
 
 using namespace tk;
@@ -254,11 +287,73 @@ extern "C" int tk_per_token_cast(const void *x, int x_dtype, int64_t M, int64_t 
     p.tiles_k = (int)((K + kStripCols - 1) / kStripCols);
     p.round_sf = round_sf;
     p.mode = mode;
+    p.xsf = SfRef{nullptr, 0, TK_SF_ROW_F32, 0, 0};
+    p.in_bm = p.in_bk = 1;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e;
     if (x_dtype == TK_BF16)
         e = fmt == TK_E4M3 ? launch_per_token<bf16_t, TK_E4M3>(p, group, s) : launch_per_token<bf16_t, TK_E2M1>(p, group, s);
     else
         e = fmt == TK_E4M3 ? launch_per_token<float, TK_E4M3>(p, group, s) : launch_per_token<float, TK_E2M1>(p, group, s);
+    return (int)e;
+}
+
+extern "C" int tk_check_per_token_cast_quantized(const void *x, int x_fmt, int64_t M, int64_t K, int64_t x_row_stride,
+                                                 const void *x_sf, int64_t x_sf_ld, int x_sf_layout, int x_bm, int x_bk,
+                                                 const void *out, const void *sf, int64_t sf_ld, int fmt, int group,
+                                                 int sf_layout, int round_sf) {
+    if (x_fmt != TK_E4M3 && x_fmt != TK_E2M1) return TK_ERR_BAD_DTYPE;
+    if (fmt != TK_E4M3 && fmt != TK_E2M1) return TK_ERR_BAD_FORMAT;
+    if (sf_layout < TK_SF_ROW_F32 || sf_layout > TK_SF_COL_UE8M0) return TK_ERR_BAD_LAYOUT;
+    if (x_sf_layout < TK_SF_ROW_F32 || x_sf_layout > TK_SF_COL_UE8M0) return TK_ERR_BAD_LAYOUT;
+    if (sf_layout == TK_SF_COL_UE8M0 && !round_sf) return TK_ERR_BAD_LAYOUT;
+    if (M < 0 || K <= 0 || K % 8 != 0) return TK_ERR_BAD_SHAPE;
+    if (M > INT32_MAX - 64 || K > INT32_MAX - 4096) return TK_ERR_TOO_LARGE;
+    if (group != 16 && group != 32 && group != 64 && group != 128) return TK_ERR_BAD_GROUP;
+    if (x_bm < 1 || x_bk < 8 || x_bk % 8 != 0) return TK_ERR_BAD_GROUP;
+    if (M == 0) return TK_OK;
+    if (!x || !x_sf || !out || !sf) return TK_ERR_NULL_POINTER;
+    if (x_row_stride < K) return TK_ERR_BAD_STRIDE;
+    const uintptr_t unit = x_fmt == TK_E4M3 ? 8 : 4;     // bytes a lane loads
+    if (!aligned_to(x, unit) || x_row_stride % 8 != 0) return TK_ERR_MISALIGNED;
+    if (!aligned_to(out, 8) || !aligned_to(sf, 4)) return TK_ERR_MISALIGNED;
+    if (x_sf_layout != TK_SF_COL_UE8M0 && !aligned_to(x_sf, 4)) return TK_ERR_MISALIGNED;
+    const int64_t nk = (K + group - 1) / group;
+    if (M * nk > INT32_MAX) return TK_ERR_TOO_LARGE;
+    const int64_t need = sf_layout == TK_SF_ROW_F32 ? nk : (sf_layout == TK_SF_COL_F32 ? M : 4 * M);
+    if (sf_ld < need) return TK_ERR_BAD_STRIDE;
+    if (sf_layout == TK_SF_COL_UE8M0 && sf_ld % 4 != 0) return TK_ERR_MISALIGNED;
+    const int64_t xnm = (M + x_bm - 1) / x_bm, xnk = (K + x_bk - 1) / x_bk;
+    const int64_t xneed = x_sf_layout == TK_SF_ROW_F32 ? xnk : (x_sf_layout == TK_SF_COL_F32 ? xnm : 4 * xnm);
+    if (x_sf_ld < xneed) return TK_ERR_BAD_STRIDE;
+    return TK_OK;
+}
+
+extern "C" int tk_per_token_cast_quantized(const void *x, int x_fmt, int64_t M, int64_t K, int64_t x_row_stride,
+                                           const void *x_sf, int64_t x_sf_ld, int x_sf_layout, int x_bm, int x_bk,
+                                           void *out, void *sf, int64_t sf_ld, int fmt, int group, int sf_layout,
+                                           int round_sf, void *stream) {
+    const int rc = tk_check_per_token_cast_quantized(x, x_fmt, M, K, x_row_stride, x_sf, x_sf_ld, x_sf_layout, x_bm, x_bk,
+                                                     out, sf, sf_ld, fmt, group, sf_layout, round_sf);
+    if (rc != TK_OK || M == 0) return rc;
+    PerTokenParams p;
+    p.x = x;
+    p.out = static_cast<uint8_t *>(out);
+    p.sf = SfRef{sf, sf_ld, sf_layout, (int)M, (int)((K + group - 1) / group)};
+    p.x_ld = x_row_stride;
+    p.M = (int)M;
+    p.K = (int)K;
+    p.tiles_k = 0;
+    p.round_sf = round_sf;
+    p.mode = TK_CAST_AND_SF;
+    p.xsf = SfRef{const_cast<void *>(x_sf), x_sf_ld, x_sf_layout, (int)((M + x_bm - 1) / x_bm), (int)((K + x_bk - 1) / x_bk)};
+    p.in_bm = x_bm;
+    p.in_bk = x_bk;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (x_fmt == TK_E4M3)
+        e = fmt == TK_E4M3 ? launch_per_token_requant<e4m3in_t, TK_E4M3>(p, group, s) : launch_per_token_requant<e4m3in_t, TK_E2M1>(p, group, s);
+    else
+        e = fmt == TK_E4M3 ? launch_per_token_requant<e2m1in_t, TK_E4M3>(p, group, s) : launch_per_token_requant<e2m1in_t, TK_E2M1>(p, group, s);
     return (int)e;
 }

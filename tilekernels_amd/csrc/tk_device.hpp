@@ -24,6 +24,19 @@ inline int wide_tile_waves(int strips) {
 }
 
 struct bf16_t { uint16_t bits; };
+struct e4m3in_t {};   // input that is itself E4M3 codes with block scales
+struct e2m1in_t {};   // input that is packed E2M1 codes (two per byte) with block scales
+
+template <typename T> struct Elem { static constexpr int bits = 8 * (int)sizeof(T); static constexpr bool quantised = false; };
+template <> struct Elem<e4m3in_t> { static constexpr int bits = 8; static constexpr bool quantised = true; };
+template <> struct Elem<e2m1in_t> { static constexpr int bits = 4; static constexpr bool quantised = true; };
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+// address of element (row, col) of a matrix with `ld` logical elements per row
+template <typename T> __device__ __forceinline__ const void *elem_ptr(const void *base, int64_t row, int64_t ld, int col) {
+    return reinterpret_cast<const uint8_t *>(base) + (((row * ld + col) * Elem<T>::bits) >> 3);
+}
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -67,13 +80,13 @@ __device__ __forceinline__ void st_stream4(void *p, uint32_t v) {
 template <typename T> struct Raw8;
 template <> struct Raw8<bf16_t> {
     u32x4 w;
-    __device__ __forceinline__ void load(const bf16_t *p) { w = ld_stream16(p); }
-    __device__ __forceinline__ void load(const bf16_t *p, bool ok) {
+    __device__ __forceinline__ void load(const void *p) { w = ld_stream16(p); }
+    __device__ __forceinline__ void load(const void *p, bool ok) {
         w = u32x4{0u, 0u, 0u, 0u};
         if (ok) w = ld_stream16(p);
     }
     // ordinary (cacheable) load, for data that is read again shortly
-    __device__ __forceinline__ void load_cached(const bf16_t *p) { w = *reinterpret_cast<const u32x4 *>(p); }
+    __device__ __forceinline__ void load_cached(const void *p) { w = *reinterpret_cast<const u32x4 *>(p); }
     __device__ __forceinline__ void zero() { w = u32x4{0u, 0u, 0u, 0u}; }
     __device__ __forceinline__ void get(float (&v)[8]) const {
         v[0] = u2f(w.x << 16); v[1] = u2f(w.x & 0xFFFF0000u);
@@ -84,19 +97,53 @@ template <> struct Raw8<bf16_t> {
 };
 template <> struct Raw8<float> {
     u32x4 a, b;
-    __device__ __forceinline__ void load(const float *p) { a = ld_stream16(p); b = ld_stream16(p + 4); }
-    __device__ __forceinline__ void load(const float *p, bool ok) {
+    __device__ __forceinline__ void load(const void *p) { a = ld_stream16(p); b = ld_stream16(reinterpret_cast<const float *>(p) + 4); }
+    __device__ __forceinline__ void load(const void *p, bool ok) {
         zero();
-        if (ok) { a = ld_stream16(p); b = ld_stream16(p + 4); }
+        if (ok) load(p);
     }
-    __device__ __forceinline__ void load_cached(const float *p) {
+    __device__ __forceinline__ void load_cached(const void *p) {
         a = *reinterpret_cast<const u32x4 *>(p);
-        b = *reinterpret_cast<const u32x4 *>(p + 4);
+        b = *(reinterpret_cast<const u32x4 *>(p) + 1);
     }
     __device__ __forceinline__ void zero() { a = u32x4{0u, 0u, 0u, 0u}; b = a; }
     __device__ __forceinline__ void get(float (&v)[8]) const {
         v[0] = u2f(a.x); v[1] = u2f(a.y); v[2] = u2f(a.z); v[3] = u2f(a.w);
         v[4] = u2f(b.x); v[5] = u2f(b.y); v[6] = u2f(b.z); v[7] = u2f(b.w);
+    }
+};
+
+// Quantised inputs: 8 codes plus the dequantisation scale of the block they sit in (`s`, set by the
+// caller); get() yields code * s, one rounding, as in the reference's dequantise-then-cast
+// (tile_kernels/torch/cast.py:87-99).
+template <> struct Raw8<e4m3in_t> {
+    u32x2 w;
+    float s;
+    __device__ __forceinline__ void load(const void *p) { w = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p)); }
+    __device__ __forceinline__ void load(const void *p, bool ok) {
+        w = u32x2{0u, 0u};
+        if (ok) load(p);
+    }
+    __device__ __forceinline__ void get(float (&v)[8]) const {
+        const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.x, false), b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.x, true);
+        const f32x2 c = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.y, false), d = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.y, true);
+        v[0] = a.x * s; v[1] = a.y * s; v[2] = b.x * s; v[3] = b.y * s;
+        v[4] = c.x * s; v[5] = c.y * s; v[6] = d.x * s; v[7] = d.y * s;
+    }
+};
+template <> struct Raw8<e2m1in_t> {
+    uint32_t w;
+    float s;
+    __device__ __forceinline__ void load(const void *p) { w = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p)); }
+    __device__ __forceinline__ void load(const void *p, bool ok) {
+        w = 0u;
+        if (ok) load(p);
+    }
+    __device__ __forceinline__ void get(float (&v)[8]) const {
+        const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1);
+        const f32x2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3);
+        v[0] = a.x * s; v[1] = a.y * s; v[2] = b.x * s; v[3] = b.y * s;
+        v[4] = c.x * s; v[5] = c.y * s; v[6] = d.x * s; v[7] = d.y * s;
     }
 };
 

@@ -16,7 +16,9 @@ def per_token_cast_impl(x, fmt, num_per_channels, x_block_size=None, use_tma_ali
                         round_sf=False, use_packed_ue8m0=False, sf_only=False, sf=None):
     assert fmt in ('e5m6', 'e4m3', 'e2m1')
     if isinstance(x, tuple):
-        raise NotImplementedError('re-quantising an already quantised (data, sf) input is not implemented')
+        assert not sf_only and sf is None
+        return _per_token_cast_quantised_input(x, fmt, num_per_channels, x_block_size, use_tma_aligned_col_major_sf,
+                                               round_sf, use_packed_ue8m0)
     assert x_block_size is None
     assert isinstance(x, torch.Tensor) and x.dtype in (torch.bfloat16, torch.float32)
     out_config = get_cast_output_config(fmt, (1, num_per_channels), use_tma_aligned_col_major_sf, round_sf, use_packed_ue8m0)
@@ -54,6 +56,53 @@ def per_token_cast_impl(x, fmt, num_per_channels, x_block_size=None, use_tma_ali
         return out
     out_sf = cast_epilogue(out_sf, num_tokens, hidden, out_config)
     return out_sf if sf_only else (out, out_sf)
+
+
+def _input_sf_storage(x_sf: torch.Tensor):
+    """(storage tensor, layout code, leading dimension) of the scale tensor of a quantised input, told
+    apart the way the reference does (tile_kernels/quant/common.py:72-82): unit stride along the rows
+    means the column-major layout, int32 elements mean packed UE8M0 bytes."""
+    assert x_sf.dim() == 2
+    if x_sf.stride(0) == 1:
+        store = x_sf.T
+        if x_sf.dtype == torch.int32:
+            store = store.view(torch.uint8)
+            return store, _ffi.TK_SF_COL_UE8M0, sf_leading_dim(store)
+        assert x_sf.dtype == torch.float32
+        return store, _ffi.TK_SF_COL_F32, sf_leading_dim(store)
+    assert x_sf.stride(1) == 1 and x_sf.dtype == torch.float32
+    return x_sf, _ffi.TK_SF_ROW_F32, sf_leading_dim(x_sf)
+
+
+def _per_token_cast_quantised_input(x, fmt, num_per_channels, x_block_size, use_tma_aligned_col_major_sf, round_sf,
+                                    use_packed_ue8m0):
+    """``x = (data, sf)``: FP8 / packed FP4 codes with one scale per ``x_block_size`` block are
+    dequantised and re-quantised in one pass (tile_kernels/quant/per_token_cast_kernel.py:87-126)."""
+    assert isinstance(x_block_size, tuple) and len(x_block_size) == 2
+    data, x_sf = x
+    assert isinstance(data, torch.Tensor) and isinstance(x_sf, torch.Tensor)
+    assert data.dtype in (torch.float8_e4m3fn, torch.int8, torch.uint8)
+    assert data.dim() == 2 and (data.stride(1) == 1 or data.shape[1] <= 1)
+    in_fp4 = data.dtype != torch.float8_e4m3fn
+    num_tokens = data.shape[0]
+    hidden = data.shape[1] * (2 if in_fp4 else 1)                    # logical width
+    token_stride = data.stride(0) * (2 if in_fp4 else 1) if num_tokens > 1 else hidden
+    out_config = get_cast_output_config(fmt, (1, num_per_channels), use_tma_aligned_col_major_sf, round_sf, use_packed_ue8m0)
+    assert num_per_channels in (16, 32, 64, 128)
+    dev = _ffi.require_gpu(data, x_sf)
+    lib = _ffi.load()
+    out = torch.empty((num_tokens, hidden if fmt == 'e4m3' else hidden // 2), dtype=out_config.torch_dtype, device=dev)
+    out_sf = alloc_scaling_factors((num_tokens, hidden), out_config, dev)
+    if num_tokens > 0:
+        store, layout, ld = _input_sf_storage(x_sf)
+        with torch.cuda.device(dev):
+            rc = lib.tk_per_token_cast_quantized(
+                data.data_ptr(), _ffi.TK_E2M1 if in_fp4 else _ffi.TK_E4M3, num_tokens, hidden, token_stride,
+                store.data_ptr(), ld, layout, x_block_size[0], x_block_size[1],
+                out.data_ptr(), out_sf.data_ptr(), sf_leading_dim(out_sf), out_config.fmt_code, num_per_channels,
+                out_config.layout_code, int(round_sf), _ffi.current_stream(dev))
+        _ffi.check(rc, 'tk_per_token_cast_quantized')
+    return out, cast_epilogue(out_sf, num_tokens, hidden, out_config)
 
 
 def per_token_cast(
