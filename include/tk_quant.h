@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define TK_QUANT_VERSION 101 /* major*10000 + minor*100 + patch */
+#define TK_QUANT_VERSION 102 /* major*10000 + minor*100 + patch */
 
 enum tk_dtype { TK_BF16 = 0, TK_F32 = 1 };
 enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1 };
@@ -143,6 +143,19 @@ int tk_check_swiglu_per_token_cast(const void *x, int x_dtype, int64_t R, int64_
                                    const int32_t *pos_to_token_topk, const float *topk_weights, int64_t num_weights,
                                    const int32_t *pos_to_expert, int use_clamp, float clamp,
                                    const int64_t *clamped_count);
+
+/*
+ * Dequantisation: out[m, k] = float(code[m, k]) * sf[m / bm, k / bk] (one fp32 product), stored as
+ * fp32 or rounded to bf16 (nearest even).  x: E4M3 bytes [M, K] or packed E2M1 bytes [M, K/2],
+ * contiguous (K in logical elements); x_sf in any of the three layouts.
+ * Stands behind tile_kernels.quant.cast_back and per_token_cast_back
+ * (tile_kernels/quant/cast_back_kernel.py:77-143).
+ *   requirements K % 8 == 0, bk % 8 == 0; out 16-byte aligned; x 8-byte (E4M3) / 4-byte (E2M1) aligned
+ */
+int tk_cast_back(const void *x, int x_fmt, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld, int x_sf_layout,
+                 int bm, int bk, void *out, int out_dtype, void *stream);
+int tk_check_cast_back(const void *x, int x_fmt, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld,
+                       int x_sf_layout, int bm, int bk, const void *out, int out_dtype);
 
 /* Text for a tk_status value (or "hip error" for positive codes). Never NULL. */
 const char *tk_strerror(int status);

@@ -205,3 +205,36 @@ def test_per_token_cast_of_quantised_input(M, K, N, x_block, in_fmt, fmt, mode):
     codes, sf = tk.quant.per_token_cast(qg, fmt, N, x_block_size=x_block, **kw)
     assert_same(codes, want_codes, 'codes')
     assert_same(sf, want_sf, 'sf')
+
+
+@pytest.mark.parametrize('out_fmt', ['bf16', 'fp32'])
+@pytest.mark.parametrize('mode', [(False, False, False), (False, True, False), (True, True, False), (True, True, True)], ids=_mode_id)
+@pytest.mark.parametrize('fmt', ['e4m3', 'e2m1'])
+@pytest.mark.parametrize('M,K,block', [(401, 7168, (1, 128)), (401, 7168, (1, 32)), (37, 576, (1, 64)), (130, 2048, (128, 128)),
+                                       (257, 2560, (32, 32)), (19, 3072, (1, 3072)), (4096, 512, (1, 128)), (1, 64, (1, 64))])
+def test_cast_back(M, K, block, fmt, mode, out_fmt):
+    """Dequantisation against the oracle, bit for bit, every scale layout; structure follows the
+    reference's tests/quant/test_cast_back.py."""
+    tk = _tk()
+    col, rnd, packed = mode
+    x = _rand((M, K), torch.bfloat16)
+    q = torch_ref.cast(x, fmt, block, use_tma_aligned_col_major_sf=col, round_sf=rnd, use_packed_ue8m0=packed)
+    want = torch_ref.cast_back(q, out_fmt, block)
+    got = tk.quant.cast_back((q[0].cuda(), _to_gpu_like(q[1])), out_fmt, block)
+    assert_same(got, want, 'dequantised')
+    if block[0] == 1:
+        assert_same(tk.quant.per_token_cast_back((q[0].cuda(), _to_gpu_like(q[1])), out_fmt, block[1]), want, 'per-token back')
+
+
+def test_cast_then_cast_back_round_trip_on_device():
+    tk = _tk()
+    x = _rand((512, 4096), torch.bfloat16).cuda()
+    q = tk.quant.per_token_cast(x, 'e4m3', 128, use_tma_aligned_col_major_sf=True, round_sf=True, use_packed_ue8m0=True)
+    back = tk.quant.per_token_cast_back(q, 'fp32', 128)
+    tk.testing.check_bias(back.cpu(), x.float().cpu())
+    # with power-of-two scales the dequantised values are exact, so re-encoding them with the same
+    # scales gives the same codes
+    codes, sf = tk.quant.per_token_cast(x, 'e4m3', 128, round_sf=True)
+    back = tk.quant.per_token_cast_back((codes, sf), 'fp32', 128)
+    again = tk.quant.per_token_cast_with_precomputed_sf(back, 'e4m3', 128, sf=sf, round_sf=True)
+    assert torch.equal(again.view(torch.uint8), codes.view(torch.uint8))

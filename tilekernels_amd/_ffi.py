@@ -31,6 +31,8 @@ SIGNATURES = {
                                         _vp, _i32, _f32, _vp, _i32, _vp]),
     'tk_check_swiglu_per_token_cast': (_i32, [_vp, _i32, _i64, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _f32, _vp, _vp,
                                               _i64, _vp, _i32, _f32, _vp]),
+    'tk_cast_back': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _i32, _vp]),
+    'tk_check_cast_back': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _i32]),
     'tk_strerror': (ctypes.c_char_p, [_i32]),
     'tk_version': (_i32, []),
 }

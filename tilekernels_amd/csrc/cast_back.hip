@@ -1,0 +1,109 @@
+// Dequantisation of block-scaled E4M3 / packed E2M1 codes back to bf16 or fp32 for gfx950.
+//
+// out[m, k] = float(code[m, k]) * sf[m / bm, k / bk], one fp32 product, then (for bf16) one
+// round-to-nearest-even conversion (v_cvt_pk_bf16_f32).  Pure streaming: a lane takes 8 consecutive
+// codes (8 or 4 bytes), their shared scale, and writes 16 (bf16) or 32 (fp32) bytes; a workgroup of
+// 4 waves covers 8 rows x 512 columns.
+//
+// Reference semantics: tile_kernels/quant/cast_back_kernel.py:19-75 (kernel) and :77-143 (wrappers),
+// tile_kernels/torch/cast.py:40-59 (oracle).
+#include "tk_device.hpp"
+#include "tk_host.hpp"
+
+namespace tk {
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kBackRowsPerWave = 2;
+
+template <typename InT, bool OUT_F32, bool FULL>
+__global__ __launch_bounds__(kThreads) void cast_back_kernel(const void *x, void *out, void *a_sf, int64_t a_sf_ld, int M, int K,
+                                                             int tiles_k, int a_sf_layout, int nm, int nk, int bm, int bk) {
+    constexpr int RPW = kBackRowsPerWave, ROWS = kWaves * RPW;
+    const SfRef sf{a_sf, a_sf_ld, a_sf_layout, nm, nk};
+    const int tile_m = blockIdx.x / tiles_k, tile_k = blockIdx.x - tile_m * tiles_k;
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const int col = tile_k * kStripCols + lane * 8;
+    const bool col_ok = FULL || col < K;
+    const int row0 = tile_m * ROWS + wave * RPW;
+
+    Raw8<InT> raw[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+        const bool ok = col_ok && (FULL || row0 + r < M);
+        raw[r].load(elem_ptr<InT>(x, row0 + r, K, col), ok);
+        raw[r].s = ok ? sf_load(sf, (row0 + r) / bm, col / bk) : 0.0f;
+    }
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+        if (!(col_ok && (FULL || row0 + r < M))) continue;
+        float v[8];
+        raw[r].get(v);
+        const int64_t idx = (int64_t)(row0 + r) * K + col;
+        if (OUT_F32) {
+            u32x4 *o = reinterpret_cast<u32x4 *>(reinterpret_cast<float *>(out) + idx);
+            __builtin_nontemporal_store(u32x4{f2u(v[0]), f2u(v[1]), f2u(v[2]), f2u(v[3])}, o);
+            __builtin_nontemporal_store(u32x4{f2u(v[4]), f2u(v[5]), f2u(v[6]), f2u(v[7])}, o + 1);
+        } else {
+            u32x4 w;
+            w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[0], v[1]}), bf16x2));
+            w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[2], v[3]}), bf16x2));
+            w.z = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[4], v[5]}), bf16x2));
+            w.w = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[6], v[7]}), bf16x2));
+            __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(out) + idx));
+        }
+    }
+}
+
+template <typename InT, bool OUT_F32>
+static hipError_t launch_cast_back(const void *x, void *out, const void *sf, int64_t sf_ld, int M, int K, int sf_layout,
+                                   int bm, int bk, hipStream_t stream) {
+    constexpr int ROWS = kWaves * kBackRowsPerWave;
+    const int tiles_m = (M + ROWS - 1) / ROWS, tiles_k = (K + kStripCols - 1) / kStripCols;
+    const int nm = (M + bm - 1) / bm, nk = (K + bk - 1) / bk;
+    const dim3 grid((unsigned)(tiles_m * tiles_k)), block(kThreads);
+    void *sfp = const_cast<void *>(sf);
+    if (M % ROWS == 0 && K % kStripCols == 0)
+        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, true>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, tiles_k, sf_layout, nm, nk, bm, bk);
+    else
+        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, false>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, tiles_k, sf_layout, nm, nk, bm, bk);
+    return hipGetLastError();
+}
+
+}  // namespace tk
+
+using namespace tk;
+
+extern "C" int tk_check_cast_back(const void *x, int x_fmt, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld,
+                                  int x_sf_layout, int bm, int bk, const void *out, int out_dtype) {
+    if (x_fmt != TK_E4M3 && x_fmt != TK_E2M1) return TK_ERR_BAD_FORMAT;
+    if (out_dtype != TK_BF16 && out_dtype != TK_F32) return TK_ERR_BAD_DTYPE;
+    if (x_sf_layout < TK_SF_ROW_F32 || x_sf_layout > TK_SF_COL_UE8M0) return TK_ERR_BAD_LAYOUT;
+    if (M < 0 || K <= 0 || K % 8 != 0) return TK_ERR_BAD_SHAPE;
+    if (M > INT32_MAX - 64 || K > INT32_MAX - 1024) return TK_ERR_TOO_LARGE;
+    if (bm < 1 || bk < 8 || bk % 8 != 0) return TK_ERR_BAD_GROUP;
+    if (M == 0) return TK_OK;
+    if (!x || !x_sf || !out) return TK_ERR_NULL_POINTER;
+    if (!aligned_to(x, x_fmt == TK_E4M3 ? 8 : 4) || !aligned_to(out, 16)) return TK_ERR_MISALIGNED;
+    if (x_sf_layout != TK_SF_COL_UE8M0 && !aligned_to(x_sf, 4)) return TK_ERR_MISALIGNED;
+    const int64_t nm = (M + bm - 1) / bm, nk = (K + bk - 1) / bk;
+    const int64_t need = x_sf_layout == TK_SF_ROW_F32 ? nk : (x_sf_layout == TK_SF_COL_F32 ? nm : 4 * nm);
+    if (x_sf_ld < need) return TK_ERR_BAD_STRIDE;
+    if (((M + 7) / 8) * ((K + kStripCols - 1) / kStripCols) > INT32_MAX) return TK_ERR_TOO_LARGE;
+    return TK_OK;
+}
+
+extern "C" int tk_cast_back(const void *x, int x_fmt, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld,
+                            int x_sf_layout, int bm, int bk, void *out, int out_dtype, void *stream) {
+    const int rc = tk_check_cast_back(x, x_fmt, M, K, x_sf, x_sf_ld, x_sf_layout, bm, bk, out, out_dtype);
+    if (rc != TK_OK || M == 0) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (x_fmt == TK_E4M3)
+        e = out_dtype == TK_F32 ? launch_cast_back<e4m3in_t, true>(x, out, x_sf, x_sf_ld, (int)M, (int)K, x_sf_layout, bm, bk, s)
+                                : launch_cast_back<e4m3in_t, false>(x, out, x_sf, x_sf_ld, (int)M, (int)K, x_sf_layout, bm, bk, s);
+    else
+        e = out_dtype == TK_F32 ? launch_cast_back<e2m1in_t, true>(x, out, x_sf, x_sf_ld, (int)M, (int)K, x_sf_layout, bm, bk, s)
+                                : launch_cast_back<e2m1in_t, false>(x, out, x_sf, x_sf_ld, (int)M, (int)K, x_sf_layout, bm, bk, s);
+    return (int)e;
+}
