@@ -12,6 +12,11 @@
 #include "tk_device.hpp"
 #include "tk_host.hpp"
 
+// Hook for timeline instrumentation in experiments; expands to nothing in the library.
+#ifndef TK_TRACE
+#define TK_TRACE(point)
+#endif
+
 namespace tk {
 
 struct SwigluParams {
@@ -156,6 +161,7 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_c
         const int row0 = tile_m * ROWS + srow;
         const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * (2 * (int64_t)p.H) + col;
 
+        TK_TRACE(0);
         Raw8<InT> rg[RPW], ru[RPW];
         bool live[RPW];   // wave-uniform
 #pragma unroll
@@ -172,6 +178,7 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_c
             }
         }
 
+        TK_TRACE(1);
         // dead rows hold zeros, so they flow through as v = 0 and only their scale is overridden
         float v[RPW][8], amax[RPW];
 #pragma unroll
@@ -220,6 +227,7 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_c
         for (int r = 0; r < RPW; ++r)
             if (col_ok && (FULL || row0 + r < p.R))
                 quantise_store8<TK_E4M3, false>(v[r], rs.inv[r], p.out + (int64_t)(row0 + r) * p.H, col);
+        TK_TRACE(2);
         __syncthreads();
         if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
         else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
