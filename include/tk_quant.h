@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define TK_QUANT_VERSION 102 /* major*10000 + minor*100 + patch */
+#define TK_QUANT_VERSION 103 /* major*10000 + minor*100 + patch */
 
 enum tk_dtype { TK_BF16 = 0, TK_F32 = 1 };
 enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1 };
@@ -156,6 +156,47 @@ int tk_cast_back(const void *x, int x_fmt, int64_t M, int64_t K, const void *x_s
                  int bm, int bk, void *out, int out_dtype, void *stream);
 int tk_check_cast_back(const void *x, int x_fmt, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld,
                        int x_sf_layout, int bm, int bk, const void *out, int out_dtype);
+
+/*
+ * Expert-major MoE layout (the step before the fused SwiGLU op in an MoE layer).
+ *
+ * tk_get_fused_mapping: stable counting sort of the flat (token, k) list by expert id (entries < 0 are
+ * skipped); expert e occupies positions [expert_start[e], expert_end[e]), its length padded to a
+ * multiple of `alignment`.  Outputs (int32): pos_to_expert / pos_to_token / pos_to_token_topk
+ * [num_expanded] (-1 on padding), token_topk_to_pos [num_tokens * num_topk] (-1 where skipped),
+ * expert_start / expert_end / num_tokens_per_expert [num_experts] (padded lengths).  Positions
+ * inside an expert follow the flat index.  `workspace` is caller-provided scratch of at least
+ * tk_fused_mapping_workspace_bytes() bytes; positions >= num_expanded are not written.
+ * Stands behind tile_kernels.moe.get_fused_mapping (tile_kernels/moe/get_fused_mapping_kernel.py:166-250).
+ *   requirements num_experts <= 1024
+ */
+int64_t tk_fused_mapping_workspace_bytes(int64_t num_tokens, int num_topk, int num_experts);
+int tk_get_fused_mapping(const int64_t *topk_idx, int64_t num_tokens, int num_topk, int num_experts, int alignment,
+                         int64_t num_expanded, int32_t *pos_to_expert, int32_t *pos_to_token, int32_t *pos_to_token_topk,
+                         int32_t *token_topk_to_pos, int32_t *expert_start, int32_t *expert_end,
+                         int32_t *num_tokens_per_expert, void *workspace, int64_t workspace_bytes, void *stream);
+int tk_check_get_fused_mapping(const int64_t *topk_idx, int64_t num_tokens, int num_topk, int num_experts, int alignment,
+                               int64_t num_expanded, const int32_t *pos_to_expert, const int32_t *pos_to_token,
+                               const int32_t *pos_to_token_topk, const int32_t *token_topk_to_pos,
+                               const int32_t *expert_start, const int32_t *expert_end,
+                               const int32_t *num_tokens_per_expert, const void *workspace, int64_t workspace_bytes);
+
+/*
+ * tk_expand_to_fused: row t of x (row_bytes bytes, any element type) is copied to every position
+ * token_topk_to_pos[t * num_topk + k] >= 0; rows with pos_to_expert < 0 are zero-filled.  With
+ * x_sf != NULL the token's `sf_cols` 4-byte scale words (contiguous rows) are expanded the same way
+ * into out_sf: row-major (word (p, j) at out_sf[p * out_sf_ld + j]) or column-major
+ * (out_sf[j * out_sf_ld + p]).
+ * Stands behind tile_kernels.moe.expand_to_fused and expand_to_fused_with_sf
+ * (tile_kernels/moe/expand_to_fused_kernel.py:94-200).
+ *   requirements row_bytes % 16 == 0; x, out 16-byte aligned
+ */
+int tk_expand_to_fused(const void *x, int64_t num_tokens, int64_t row_bytes, const int32_t *token_topk_to_pos, int num_topk,
+                       const int32_t *pos_to_expert, int64_t num_expanded, void *out, const void *x_sf, int sf_cols,
+                       void *out_sf, int64_t out_sf_ld, int sf_col_major, void *stream);
+int tk_check_expand_to_fused(const void *x, int64_t num_tokens, int64_t row_bytes, const int32_t *token_topk_to_pos,
+                             int num_topk, const int32_t *pos_to_expert, int64_t num_expanded, const void *out,
+                             const void *x_sf, int sf_cols, const void *out_sf, int64_t out_sf_ld, int sf_col_major);
 
 /* Text for a tk_status value (or "hip error" for positive codes). Never NULL. */
 const char *tk_strerror(int status);

@@ -300,3 +300,79 @@ def swiglu_forward_and_per_token_cast(
         codes.view(torch.uint8).masked_fill_(dead, 0)
         sf.masked_fill_(dead, 0)          # in place: keeps the column-major strides
     return codes, sf
+
+
+# --------------------------------------------------------------------------------------------------
+# MoE expert-major ("fused") layout: the callers on either side of the fused SwiGLU op.
+
+def get_fused_mapping(topk_idx: torch.Tensor, num_experts: int, alignment: int):
+    """Maps between the (token, k) list and the expert-major expanded layout.
+
+    Contract of tile_kernels.moe.get_fused_mapping (tile_kernels/moe/get_fused_mapping_kernel.py:166-250)
+    as its test states it (tests/moe/test_get_fused_mapping.py:54-78): experts occupy consecutive
+    segments, each padded to a multiple of ``alignment`` rows; padding positions hold -1.  The
+    reference leaves the order inside a segment unspecified; this statement fixes it as the order of
+    the flat (token, k) index (a stable counting sort).
+
+    Returns (pos_to_expert, pos_to_token, pos_to_token_topk, token_topk_to_pos, expert_start, expert_end,
+    num_tokens_per_expert), all int32; num_tokens_per_expert holds the padded segment lengths.
+    """
+    assert topk_idx.dim() == 2
+    num_tokens, num_topk = topk_idx.shape
+    flat = topk_idx.reshape(-1).to(torch.int64)
+    live = flat >= 0
+    counts = torch.bincount(flat[live], minlength=num_experts)
+    padded = (counts + alignment - 1) // alignment * alignment
+    ends = torch.cumsum(padded, 0)
+    starts = ends - padded
+    total = int(ends[-1]) if num_experts else 0
+    pos_to_expert = torch.full((total,), -1, dtype=torch.int32)
+    pos_to_token = torch.full((total,), -1, dtype=torch.int32)
+    pos_to_token_topk = torch.full((total,), -1, dtype=torch.int32)
+    token_topk_to_pos = torch.full((num_tokens * num_topk,), -1, dtype=torch.int32)
+    idx = torch.nonzero(live).flatten()
+    order = idx[torch.argsort(flat[idx], stable=True)]          # grouped by expert, flat index ascending inside
+    experts = flat[order]
+    rank = torch.arange(order.numel()) - (torch.cumsum(counts, 0) - counts)[experts]
+    pos = starts[experts] + rank
+    pos_to_expert[pos] = experts.to(torch.int32)
+    pos_to_token[pos] = (order // num_topk).to(torch.int32)
+    pos_to_token_topk[pos] = order.to(torch.int32)
+    token_topk_to_pos[order] = pos.to(torch.int32)
+    return (pos_to_expert, pos_to_token, pos_to_token_topk, token_topk_to_pos.view(num_tokens, num_topk),
+            starts.to(torch.int32), ends.to(torch.int32), padded.to(torch.int32))
+
+
+def expand_to_fused(x: torch.Tensor, token_topk_to_pos: torch.Tensor, pos_to_expert: torch.Tensor) -> torch.Tensor:
+    """Row t of ``x`` is copied to every position token_topk_to_pos[t, k] >= 0; all other rows of the
+    expanded tensor are zero (tile_kernels/torch/expand_to_fused.py:6-39)."""
+    num_tokens, hidden = x.shape
+    out = torch.zeros((pos_to_expert.shape[0], hidden), dtype=x.dtype)
+    num_topk = token_topk_to_pos.shape[1]
+    pos = token_topk_to_pos.reshape(-1).long()
+    src = torch.arange(num_tokens).repeat_interleave(num_topk)
+    keep = pos >= 0
+    as_bytes = out.view(torch.uint8)                 # index_copy on raw bytes: works for fp8 / int8 alike
+    as_bytes[pos[keep]] = x.view(torch.uint8)[src[keep]]
+    return out
+
+
+def expand_to_fused_with_sf(x: QuantTensor, num_per_channels: int, token_topk_to_pos: torch.Tensor,
+                            pos_to_expert: torch.Tensor, use_tma_aligned_col_major_sf: bool = False):
+    """Same expansion for codes and their row-major scale rows; the expanded scales come back
+    row-major, or column-major over a 4-row-aligned buffer (tile_kernels/torch/expand_to_fused.py:42-91)."""
+    data, sf = x
+    out = expand_to_fused(data, token_topk_to_pos, pos_to_expert)
+    num_expanded = pos_to_expert.shape[0]
+    cols = sf.shape[1]
+    if use_tma_aligned_col_major_sf:
+        store = torch.zeros((cols, _round_up(num_expanded, 4)), dtype=sf.dtype)
+        out_sf = store[:, :num_expanded].T
+    else:
+        out_sf = torch.zeros((num_expanded, cols), dtype=sf.dtype)
+    num_topk = token_topk_to_pos.shape[1]
+    pos = token_topk_to_pos.reshape(-1).long()
+    src = torch.arange(data.shape[0]).repeat_interleave(num_topk)
+    keep = pos >= 0
+    out_sf[pos[keep]] = sf[src[keep]]
+    return out, out_sf

@@ -1,0 +1,260 @@
+// Expert-major ("fused") MoE layout for gfx950: the mapping between the (token, k) routing list and
+// the expanded row order, and the row expansion that feeds the fused SwiGLU op.  Integer / byte
+// work, HBM- and latency-bound; no LDS tiling beyond per-wave histograms.
+//
+// Reference semantics: tile_kernels/moe/get_fused_mapping_kernel.py:24-250,
+// tile_kernels/moe/expand_to_fused_kernel.py:16-200, tile_kernels/torch/expand_to_fused.py.
+#include "tk_device.hpp"
+#include "tk_host.hpp"
+
+namespace tk {
+
+// ------------------------------------------------------------------------------------------------
+// get_fused_mapping: a stable counting sort of the flat (token, k) list by expert, every expert's
+// segment padded to a multiple of `alignment`.  Three launches, no grid-wide barrier:
+//   count  : each wave histograms its own 256-element slice            -> ws[slice][expert]
+//   scan   : one workgroup turns the histograms into exclusive offsets  -> ws[slice][expert], expert_start/end
+//   assign : each wave walks its slice again in order and hands out positions
+// Positions inside an expert follow the flat index (the reference leaves that order open).
+constexpr int kSliceElems = 256;   // elements per wave
+constexpr int kMaxExperts = 1024;  // bound on the per-wave LDS histogram
+
+__global__ __launch_bounds__(kThreads) void fused_mapping_count_kernel(const int64_t *topk_idx, int numel, int num_experts,
+                                                                       int32_t *ws, int32_t *pos_to_expert, int32_t *pos_to_token,
+                                                                       int32_t *pos_to_token_topk, int num_expanded) {
+    extern __shared__ int32_t hist[];   // [kWaves][num_experts]
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const int slice = blockIdx.x * kWaves + wave;
+    int32_t *h = hist + wave * num_experts;
+    for (int e = lane; e < num_experts; e += 64) h[e] = 0;
+    // padding positions keep -1; the assign launch overwrites the live ones
+    for (int i = blockIdx.x * kThreads + threadIdx.x; i < num_expanded; i += gridDim.x * kThreads) {
+        pos_to_expert[i] = -1;
+        pos_to_token[i] = -1;
+        pos_to_token_topk[i] = -1;
+    }
+    __syncthreads();
+    const int base = slice * kSliceElems;
+    for (int j = lane; j < kSliceElems; j += 64) {
+        const int i = base + j;
+        if (i < numel) {
+            const int64_t e = topk_idx[i];
+            if (e >= 0 && e < num_experts) atomicAdd(&h[(int)e], 1);
+        }
+    }
+    __syncthreads();
+    if (base < numel)
+        for (int e = lane; e < num_experts; e += 64) ws[(int64_t)slice * num_experts + e] = h[e];
+}
+
+__global__ __launch_bounds__(1024) void fused_mapping_scan_kernel(int32_t *ws, int num_slices, int num_experts, int alignment,
+                                                                  int32_t *expert_start, int32_t *expert_end,
+                                                                  int32_t *num_tokens_per_expert) {
+    __shared__ int32_t padded[kMaxExperts];
+    __shared__ int32_t start[kMaxExperts];
+    for (int e = threadIdx.x; e < num_experts; e += blockDim.x) {
+        int32_t run = 0;
+        for (int s = 0; s < num_slices; ++s) {
+            const int64_t at = (int64_t)s * num_experts + e;
+            const int32_t c = ws[at];
+            ws[at] = run;          // exclusive offset of this slice inside the expert
+            run += c;
+        }
+        padded[e] = (run + alignment - 1) / alignment * alignment;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int32_t run = 0;
+        for (int e = 0; e < num_experts; ++e) {
+            start[e] = run;
+            run += padded[e];
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < num_experts; e += blockDim.x) {
+        expert_start[e] = start[e];
+        expert_end[e] = start[e] + padded[e];
+        num_tokens_per_expert[e] = padded[e];
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void fused_mapping_assign_kernel(const int64_t *topk_idx, int numel, int num_topk,
+                                                                        int num_experts, int expert_bits, const int32_t *ws,
+                                                                        const int32_t *expert_start, int32_t *pos_to_expert,
+                                                                        int32_t *pos_to_token, int32_t *pos_to_token_topk,
+                                                                        int32_t *token_topk_to_pos, int num_expanded) {
+    extern __shared__ int32_t next[];   // [kWaves][num_experts]: next free position per expert, per wave
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const int slice = blockIdx.x * kWaves + wave;
+    const int base = slice * kSliceElems;
+    if (base >= numel) return;          // whole wave; no barrier below
+    int32_t *nx = next + wave * num_experts;
+    for (int e = lane; e < num_experts; e += 64) nx[e] = expert_start[e] + ws[(int64_t)slice * num_experts + e];
+    __builtin_amdgcn_wave_barrier();
+    const unsigned long long below = (1ull << lane) - 1ull;
+    for (int j = 0; j < kSliceElems; j += 64) {
+        const int i = base + j + lane;
+        int e = -1;
+        if (i < numel) {
+            const int64_t v = topk_idx[i];
+            e = (v >= 0 && v < num_experts) ? (int)v : -1;
+        }
+        // lanes holding the same expert: intersect the ballots of every bit of the id
+        unsigned long long peers = __ballot(e >= 0);
+        for (int b = 0; b < expert_bits; ++b) {
+            const bool bit = (e >> b) & 1;
+            const unsigned long long m = __ballot(bit);
+            peers &= bit ? m : ~m;
+        }
+        int pos = -1;
+        if (e >= 0) {
+            const int first = nx[e];
+            pos = first + __popcll(peers & below);
+            __builtin_amdgcn_wave_barrier();          // every peer has read before the last one advances the counter
+            if ((peers >> lane) == 1ull) nx[e] = first + __popcll(peers);
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (i < numel) token_topk_to_pos[i] = pos;
+        if (pos >= 0 && pos < num_expanded) {
+            pos_to_expert[pos] = e;
+            pos_to_token[pos] = i / num_topk;
+            pos_to_token_topk[pos] = i;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// expand_to_fused: workgroup t < T copies row t to each of its positions (read once, written once
+// per destination); workgroup T + r zero-fills row r when it is padding.  Rows are moved as raw
+// 16-byte pieces, so any element type works.  Optional 4-byte scale rows travel the same way into a
+// row-major or column-major scale tensor.
+__global__ __launch_bounds__(kThreads) void expand_to_fused_kernel(const uint8_t *x, int64_t row_bytes, const int32_t *token_topk_to_pos,
+                                                                   int num_topk, const int32_t *pos_to_expert, int num_tokens,
+                                                                   int num_expanded, uint8_t *out, const uint32_t *x_sf, int sf_cols,
+                                                                   uint32_t *out_sf, int64_t out_sf_ld, int sf_col_major) {
+    const int b = blockIdx.x;
+    if (b < num_tokens) {
+        const int32_t *pos = token_topk_to_pos + (int64_t)b * num_topk;
+        const uint8_t *src = x + (int64_t)b * row_bytes;
+        for (int64_t off = (int64_t)threadIdx.x * 16; off < row_bytes; off += kThreads * 16) {
+            const u32x4 v = ld_stream16(src + off);
+            for (int k = 0; k < num_topk; ++k) {
+                const int p = uniform_load(pos + k);
+                if (p >= 0 && p < num_expanded)
+                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out + (int64_t)p * row_bytes + off));
+            }
+        }
+        if (x_sf) {
+            for (int j = threadIdx.x; j < sf_cols; j += kThreads) {
+                const uint32_t s = x_sf[(int64_t)b * sf_cols + j];
+                for (int k = 0; k < num_topk; ++k) {
+                    const int p = uniform_load(pos + k);
+                    if (p >= 0 && p < num_expanded) out_sf[sf_col_major ? (int64_t)j * out_sf_ld + p : (int64_t)p * out_sf_ld + j] = s;
+                }
+            }
+        }
+    } else {
+        const int r = b - num_tokens;
+        if (uniform_load(pos_to_expert + r) >= 0) return;
+        uint8_t *dst = out + (int64_t)r * row_bytes;
+        for (int64_t off = (int64_t)threadIdx.x * 16; off < row_bytes; off += kThreads * 16)
+            __builtin_nontemporal_store(u32x4{0u, 0u, 0u, 0u}, reinterpret_cast<u32x4 *>(dst + off));
+        if (x_sf)
+            for (int j = threadIdx.x; j < sf_cols; j += kThreads) out_sf[sf_col_major ? (int64_t)j * out_sf_ld + r : (int64_t)r * out_sf_ld + j] = 0u;
+    }
+}
+
+}  // namespace tk
+
+using namespace tk;
+
+extern "C" int64_t tk_fused_mapping_workspace_bytes(int64_t num_tokens, int num_topk, int num_experts) {
+    if (num_tokens < 0 || num_topk <= 0 || num_experts <= 0) return 0;
+    const int64_t slices = (num_tokens * num_topk + kSliceElems - 1) / kSliceElems;
+    const int64_t padded = (slices + kWaves - 1) / kWaves * kWaves;       // whole workgroups
+    return padded * num_experts * (int64_t)sizeof(int32_t);
+}
+
+extern "C" int tk_check_get_fused_mapping(const int64_t *topk_idx, int64_t num_tokens, int num_topk, int num_experts,
+                                          int alignment, int64_t num_expanded, const int32_t *pos_to_expert,
+                                          const int32_t *pos_to_token, const int32_t *pos_to_token_topk,
+                                          const int32_t *token_topk_to_pos, const int32_t *expert_start,
+                                          const int32_t *expert_end, const int32_t *num_tokens_per_expert,
+                                          const void *workspace, int64_t workspace_bytes) {
+    if (num_tokens < 0 || num_topk <= 0 || num_expanded < 0) return TK_ERR_BAD_SHAPE;
+    if (num_experts <= 0 || num_experts > kMaxExperts) return TK_ERR_BAD_GROUP;
+    if (alignment <= 0) return TK_ERR_BAD_VALUE;
+    if (num_tokens * num_topk > INT32_MAX - 1024 || num_expanded > INT32_MAX - 1024) return TK_ERR_TOO_LARGE;
+    if (!expert_start || !expert_end || !num_tokens_per_expert) return TK_ERR_NULL_POINTER;
+    if (num_tokens > 0 && (!topk_idx || !token_topk_to_pos || !workspace)) return TK_ERR_NULL_POINTER;
+    if (num_expanded > 0 && (!pos_to_expert || !pos_to_token || !pos_to_token_topk)) return TK_ERR_NULL_POINTER;
+    if (workspace_bytes < tk_fused_mapping_workspace_bytes(num_tokens, num_topk, num_experts)) return TK_ERR_BAD_STRIDE;
+    if (!aligned_to(topk_idx, 8) || !aligned_to(workspace, 4)) return TK_ERR_MISALIGNED;
+    return TK_OK;
+}
+
+extern "C" int tk_get_fused_mapping(const int64_t *topk_idx, int64_t num_tokens, int num_topk, int num_experts, int alignment,
+                                    int64_t num_expanded, int32_t *pos_to_expert, int32_t *pos_to_token,
+                                    int32_t *pos_to_token_topk, int32_t *token_topk_to_pos, int32_t *expert_start,
+                                    int32_t *expert_end, int32_t *num_tokens_per_expert, void *workspace,
+                                    int64_t workspace_bytes, void *stream) {
+    const int rc = tk_check_get_fused_mapping(topk_idx, num_tokens, num_topk, num_experts, alignment, num_expanded, pos_to_expert,
+                                              pos_to_token, pos_to_token_topk, token_topk_to_pos, expert_start, expert_end,
+                                              num_tokens_per_expert, workspace, workspace_bytes);
+    if (rc != TK_OK) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int numel = (int)(num_tokens * num_topk);
+    const int slices = (numel + kSliceElems - 1) / kSliceElems;
+    const int blocks = (slices + kWaves - 1) / kWaves;
+    int32_t *ws = static_cast<int32_t *>(workspace);
+    const size_t lds = (size_t)kWaves * num_experts * sizeof(int32_t);
+    int bits = 0;
+    while ((1 << bits) < num_experts) ++bits;
+    // the count launch also fills the padding markers, so it runs even when there are no tokens
+    const int fill_blocks = (int)((num_expanded + kThreads - 1) / kThreads);
+    const int count_grid = blocks > 0 ? blocks : (fill_blocks > 1024 ? 1024 : fill_blocks);
+    if (count_grid > 0)
+        hipLaunchKernelGGL(fused_mapping_count_kernel, dim3(count_grid), dim3(kThreads), lds, s, topk_idx, numel, num_experts, ws,
+                           pos_to_expert, pos_to_token, pos_to_token_topk, (int)num_expanded);
+    hipLaunchKernelGGL(fused_mapping_scan_kernel, dim3(1), dim3(1024), 0, s, ws, slices, num_experts, alignment, expert_start,
+                       expert_end, num_tokens_per_expert);
+    if (blocks > 0)
+        hipLaunchKernelGGL(fused_mapping_assign_kernel, dim3(blocks), dim3(kThreads), lds, s, topk_idx, numel, num_topk, num_experts,
+                           bits, ws, expert_start, pos_to_expert, pos_to_token, pos_to_token_topk, token_topk_to_pos,
+                           (int)num_expanded);
+    return (int)hipGetLastError();
+}
+
+extern "C" int tk_check_expand_to_fused(const void *x, int64_t num_tokens, int64_t row_bytes, const int32_t *token_topk_to_pos,
+                                        int num_topk, const int32_t *pos_to_expert, int64_t num_expanded, const void *out,
+                                        const void *x_sf, int sf_cols, const void *out_sf, int64_t out_sf_ld,
+                                        int sf_col_major) {
+    if (num_tokens < 0 || num_expanded < 0 || row_bytes <= 0 || num_topk <= 0) return TK_ERR_BAD_SHAPE;
+    if (row_bytes % 16 != 0) return TK_ERR_MISALIGNED;
+    if (num_tokens + num_expanded > INT32_MAX - 1024) return TK_ERR_TOO_LARGE;
+    if (num_expanded > 0 && (!pos_to_expert || !out)) return TK_ERR_NULL_POINTER;
+    if (num_tokens > 0 && (!x || !token_topk_to_pos)) return TK_ERR_NULL_POINTER;
+    if (!aligned_to(x, 16) || !aligned_to(out, 16)) return TK_ERR_MISALIGNED;
+    if (x_sf) {
+        if (sf_cols <= 0) return TK_ERR_BAD_SHAPE;
+        if (!out_sf) return TK_ERR_NULL_POINTER;
+        if (!aligned_to(x_sf, 4) || !aligned_to(out_sf, 4)) return TK_ERR_MISALIGNED;
+        if (out_sf_ld < (sf_col_major ? num_expanded : sf_cols)) return TK_ERR_BAD_STRIDE;
+    }
+    return TK_OK;
+}
+
+extern "C" int tk_expand_to_fused(const void *x, int64_t num_tokens, int64_t row_bytes, const int32_t *token_topk_to_pos,
+                                  int num_topk, const int32_t *pos_to_expert, int64_t num_expanded, void *out, const void *x_sf,
+                                  int sf_cols, void *out_sf, int64_t out_sf_ld, int sf_col_major, void *stream) {
+    const int rc = tk_check_expand_to_fused(x, num_tokens, row_bytes, token_topk_to_pos, num_topk, pos_to_expert, num_expanded, out,
+                                            x_sf, sf_cols, out_sf, out_sf_ld, sf_col_major);
+    if (rc != TK_OK) return rc;
+    const int64_t grid = num_tokens + num_expanded;
+    if (grid == 0) return TK_OK;
+    hipLaunchKernelGGL(expand_to_fused_kernel, dim3((unsigned)grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint8_t *>(x), row_bytes, token_topk_to_pos, num_topk, pos_to_expert, (int)num_tokens,
+                       (int)num_expanded, static_cast<uint8_t *>(out), static_cast<const uint32_t *>(x_sf), sf_cols,
+                       static_cast<uint32_t *>(out_sf), out_sf_ld, sf_col_major);
+    return (int)hipGetLastError();
+}
