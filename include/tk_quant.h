@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define TK_QUANT_VERSION 103 /* major*10000 + minor*100 + patch */
+#define TK_QUANT_VERSION 104 /* major*10000 + minor*100 + patch */
 
 enum tk_dtype { TK_BF16 = 0, TK_F32 = 1 };
 enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1 };
@@ -143,6 +143,35 @@ int tk_check_swiglu_per_token_cast(const void *x, int x_dtype, int64_t R, int64_
                                    const int32_t *pos_to_token_topk, const float *topk_weights, int64_t num_weights,
                                    const int32_t *pos_to_expert, int use_clamp, float clamp,
                                    const int64_t *clamped_count);
+
+/*
+ * Fused SwiGLU backward + per-token E4M3 quantisation of the input gradient.  x is the forward input as
+ * it was quantised: E4M3 codes [R, 2H] (gate = columns [0, H), up = [H, 2H)) with fp32 scales
+ * x_sf[R, 2H/group], both contiguous.  In fp32, with g = code * sf, u likewise, go = grad_out:
+ *   use_clamp: g = min(g, clamp), u = min(max(u, -clamp), clamp); the gradient of a clamped value is 0
+ *   d = 1 + exp(-g), s = 1 / d, act = g / d * u, w = topk_weights[pos_to_token_topk[r]] (0 where < 0)
+ *   out         [R, H]  bf16 = act * w
+ *   x_grad      [R, 2H] bf16 = [ go*w*s * u * fma(g, 1 - s, 1) | go*w*s * g ]
+ *   x_grad_codes[R, 2H] E4M3 with x_grad_sf[R, 2H/group] fp32 (row-major): the per-token cast of the
+ *                       fp32 gradient over groups of `group` columns (round_sf as in tk_per_token_cast)
+ *   weight_grad [num_weights] fp32 = sum over the row of go * act at index pos_to_token_topk[r] >= 0,
+ *                       and 0 at every index i with token_topk_to_pos[i] < 0
+ * Stands behind tile_kernels.quant.swiglu_backward_and_per_token_cast
+ * (tile_kernels/quant/swiglu_backward_and_per_token_cast_kernel.py:166-244).
+ *   requirements        group in {32, 128}; H % group == 0; grad_out, out, x_grad 16-byte aligned,
+ *                       x and x_grad_codes 8-byte aligned; num_weights = num_tokens * num_topk
+ */
+int tk_swiglu_backward_per_token_cast(const void *x, const float *x_sf, int64_t R, int64_t H, int group,
+                                      const void *grad_out, const float *topk_weights, const int32_t *pos_to_token_topk,
+                                      const int32_t *token_topk_to_pos, int64_t num_weights, void *out,
+                                      void *x_grad_codes, float *x_grad_sf, void *x_grad, float *weight_grad,
+                                      int round_sf, int use_clamp, float clamp, void *stream);
+int tk_check_swiglu_backward_per_token_cast(const void *x, const float *x_sf, int64_t R, int64_t H, int group,
+                                            const void *grad_out, const float *topk_weights,
+                                            const int32_t *pos_to_token_topk, const int32_t *token_topk_to_pos,
+                                            int64_t num_weights, const void *out, const void *x_grad_codes,
+                                            const float *x_grad_sf, const void *x_grad, const float *weight_grad,
+                                            int round_sf, int use_clamp, float clamp);
 
 /*
  * Dequantisation: out[m, k] = float(code[m, k]) * sf[m / bm, k / bk] (one fp32 product), stored as

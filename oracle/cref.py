@@ -35,6 +35,9 @@ def lib():
         L.tkref_swiglu.restype = i32
         L.tkref_e4m3_encode_n.argtypes = [vp, i64, vp]
         L.tkref_e2m1_encode_n.argtypes = [vp, i64, vp]
+        L.tkref_swiglu_backward.argtypes = [vp, vp, i64, i64, i32, vp, vp, i64, vp, i32, f32, vp, vp, vp]
+        L.tkref_swiglu_backward.restype = i32
+        L.tkref_fmaf_n.argtypes = [vp, vp, vp, i64, vp]
         L.tkref_count_div_mismatches.argtypes = [f32, ctypes.c_uint32, ctypes.c_uint32, i32]
         L.tkref_count_div_mismatches.restype = i64
         _lib = L
@@ -105,3 +108,32 @@ def count_div_mismatches(c: float, lo_bits: int, hi_bits: int, uncorrected: bool
     """Positive floats in [lo_bits, hi_bits) (bit patterns) where a*y + fma(-c, a*y, a)*y != a/c
     (``uncorrected``: where a*y alone != a/c)."""
     return int(lib().tkref_count_div_mismatches(c, lo_bits, hi_bits, int(uncorrected)))
+
+
+def swiglu_backward(x, grad_out: torch.Tensor, weight: torch.Tensor, pos_to_token_topk: torch.Tensor,
+                    num_per_channels: int, swiglu_clamp_value=None):
+    """Returns fp32 ``(out [R, H], x_grad [R, 2H], weight_grad like weight)``."""
+    codes, sf = x
+    codes = codes.view(torch.uint8).contiguous()
+    R, H2 = codes.shape
+    H = H2 // 2
+    sf = sf.to(torch.float32).contiguous()
+    assert grad_out.dtype == torch.bfloat16 and grad_out.is_contiguous() and tuple(grad_out.shape) == (R, H)
+    w = weight.to(torch.float32).contiguous()
+    p = pos_to_token_topk.to(torch.int32).contiguous()
+    out = torch.empty((R, H), dtype=torch.float32)
+    x_grad = torch.empty((R, H2), dtype=torch.float32)
+    w_grad = torch.empty_like(w)
+    rc = lib().tkref_swiglu_backward(_ptr(codes), _ptr(sf), R, H, num_per_channels, _ptr(grad_out), _ptr(w), w.numel(),
+                                     _ptr(p), int(swiglu_clamp_value is not None),
+                                     0.0 if swiglu_clamp_value is None else float(swiglu_clamp_value),
+                                     _ptr(out), _ptr(x_grad), _ptr(w_grad))
+    assert rc == 0
+    return out, x_grad, w_grad
+
+
+def fmaf(a: np.ndarray, b: np.ndarray, c: np.ndarray) -> np.ndarray:
+    a, b, c = (np.ascontiguousarray(t, dtype=np.float32) for t in (a, b, c))
+    out = np.empty(a.shape, dtype=np.float32)
+    lib().tkref_fmaf_n(a.ctypes.data, b.ctypes.data, c.ctypes.data, a.size, out.ctypes.data)
+    return out

@@ -4,7 +4,7 @@
  * Nothing that ships links or loads this file: only tests, the smoke check and the CPU-baseline
  * leg of the benchmark do, as the checker.  It exists as a second, independently written
  * statement of the same algorithm as oracle/torch_ref.py, so that a slip in either one shows up as
- * a bit mismatch between the two (tests/test_oracle_cross.py), and so that full-size inputs can
+ * a bit mismatch between the two (tests/test_oracle_cast.py, tests/test_oracle_swiglu_backward.py), and so that full-size inputs can
  * be checked in seconds.
  *
  * Algorithm followed (reference file:line):
@@ -12,6 +12,7 @@
  *   use of a caller-supplied scale (1/sf, clamp +-448) ............. tile_kernels/torch/cast.py:165-190
  *   E2M1 code assignment and nibble packing ....................... tile_kernels/torch/cast.py:192-196, 224-252
  *   SwiGLU g/(1+exp(-g))*u, clamp, counters, routing weight ....... tile_kernels/torch/swiglu.py:62-86
+ *   SwiGLU backward on a dequantised input ........................ tile_kernels/torch/swiglu.py:98-227
  *
  * Pins: tkref_e4m3_encode / tkref_e2m1_encode are checked against brute-force nearest-value
  * searches over the OCP value tables and hand known answers (tests/test_oracle_encoders.py); the
@@ -168,6 +169,70 @@ int tkref_swiglu(const void *x, int x_is_f32, int64_t R, int64_t H, const int32_
     }
     if (counts) { counts[0] += n0; counts[1] += n1; counts[2] += n2; }
     return 0;
+}
+
+/* OCP E4M3FN byte -> fp32 (0x7f / 0xff are NaN) */
+static inline float e4m3_decode(uint8_t c) {
+    const uint32_t e = (c >> 3) & 15u, m = c & 7u;
+    float a;
+    if (e == 15u && m == 7u) a = NAN;
+    else if (e == 0u) a = (float)m * 0x1p-9f;
+    else a = u2f(((e + 120u) << 23) | (m << 20));
+    return (c & 0x80u) ? -a : a;
+}
+
+/*
+ * SwiGLU backward on a quantised forward input (tile_kernels/torch/swiglu.py:98-227).
+ *   codes[R, 2H] E4M3 bytes, sf[R, 2H/N] fp32 (N = group), grad_out[R, H] bf16 bits,
+ *   weight[T*K] fp32, pos_to_token_topk[R] (negative = padding row, weight 0).
+ * Outputs, all fp32: out[R, H] = g/(1+exp(-g))*u*w, x_grad[R, 2H] = [d/dgate | d/dup],
+ * weight_grad[T*K] (zero-filled first, then the row dot products sum(grad_out * act)).
+ * The only fused operation is fma(g, 1 - s, 1); every other product is rounded once.
+ */
+int tkref_swiglu_backward(const uint8_t *codes, const float *sf, int64_t R, int64_t H, int group,
+                          const uint16_t *grad_out, const float *weight, int64_t num_weights,
+                          const int32_t *pos_to_token_topk, int use_clamp, float clamp, float *out,
+                          float *x_grad, float *weight_grad) {
+    if (R < 0 || H <= 0 || group <= 0 || H % group) return -1;
+    const int64_t nsf = 2 * H / group;
+    for (int64_t i = 0; i < num_weights; ++i) weight_grad[i] = 0.0f;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < R; ++r) {
+        const int32_t idx = pos_to_token_topk[r];
+        const float w = idx >= 0 ? weight[idx] : 0.0f;
+        float dot = 0.0f;
+        for (int64_t c = 0; c < H; ++c) {
+            float g = e4m3_decode(codes[r * 2 * H + c]) * sf[r * nsf + c / group];
+            float u = e4m3_decode(codes[r * 2 * H + H + c]) * sf[r * nsf + (H + c) / group];
+            int cg = 0, cu = 0;
+            if (use_clamp) {
+                cg = g > clamp;
+                if (cg) g = clamp;
+                if (u > clamp) { u = clamp; cu = 1; }
+                else if (u < -clamp) { u = -clamp; cu = 1; }
+            }
+            const float go = bf16_to_f32(grad_out[r * H + c]);
+            const float d = 1.0f + expf(-g);
+            const float s = 1.0f / d;
+            float t = go * w;
+            t = t * s;
+            float dg = t * u;
+            dg = dg * fmaf(g, 1.0f - s, 1.0f);
+            const float du = t * g;
+            float act = g / d;
+            act = act * u;
+            out[r * H + c] = act * w;
+            x_grad[r * 2 * H + c] = cg ? 0.0f : dg;
+            x_grad[r * 2 * H + H + c] = cu ? 0.0f : du;
+            dot += go * act;
+        }
+        if (idx >= 0) weight_grad[idx] = dot;
+    }
+    return 0;
+}
+
+void tkref_fmaf_n(const float *a, const float *b, const float *c, int64_t n, float *out) {
+    for (int64_t i = 0; i < n; ++i) out[i] = fmaf(a[i], b[i], c[i]);
 }
 
 /* bulk helpers so Python can test the encoders over whole arrays */

@@ -5,6 +5,7 @@ pure-torch implementations:
 
 * ``cast`` / ``cast_back``      <- tile_kernels/torch/cast.py:62-221 and :40-59
 * ``swiglu_forward``            <- tile_kernels/torch/swiglu.py:9-88
+* ``swiglu_backward``           <- tile_kernels/torch/swiglu.py:90-227
 * ``unpack_from_e2m1fn_x2``     <- tile_kernels/quant/common.py:247-295
 * ``encode_e2m1``               <- tile_kernels/torch/cast.py:224-252 (same result, closed form)
 
@@ -25,6 +26,9 @@ How each function is pinned (all pins live in tests/test_oracle_*.py and run wit
 * the whole of ``cast`` is cross-checked bit-for-bit against the independent scalar C
   restatement in oracle/quant_ref.c.
 * ``swiglu_forward`` is checked against float64 evaluation and ``torch.nn.functional.silu``.
+* ``swiglu_backward`` is checked against float64 autograd of ``silu(g) * u * w`` (a dropped term,
+  a wrong sign or swapped halves fails it), against hand-set clamp cases, and its ``fma_f32`` helper
+  against the C library's correctly rounded ``fmaf`` on operands built to hit double rounding.
 """
 from typing import Optional, Tuple, Union
 
@@ -300,6 +304,120 @@ def swiglu_forward_and_per_token_cast(
         codes.view(torch.uint8).masked_fill_(dead, 0)
         sf.masked_fill_(dead, 0)          # in place: keeps the column-major strides
     return codes, sf
+
+
+def fma_f32(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> torch.Tensor:
+    """Correctly rounded fp32 ``a * b + c`` (one rounding), elementwise.
+
+    The reference evaluates ``x * (1 - s) + 1`` through a compiled helper so that it becomes a single
+    fused multiply-add (tile_kernels/torch/swiglu.py:90-95).  Here the product of two fp32 values is
+    exact in float64 (48 significant bits); the float64 sum is then forced to round-to-odd with the
+    error term of a TwoSum, which makes the final rounding to fp32 the rounding of the exact value.
+    """
+    p = a.to(torch.float64) * b.to(torch.float64)
+    c = c.to(torch.float64).expand_as(p)
+    s = p + c
+    bb = s - p
+    err = (p - (s - bb)) + (c - bb)
+    bits = s.contiguous().view(torch.int64).clone()
+    fix = (err != 0) & torch.isfinite(s) & ((bits & 1) == 0) & (s != 0)
+    grow = (err > 0) == (s > 0)            # the exact value lies further from zero than s
+    bits = torch.where(fix, torch.where(grow, bits + 1, bits - 1), bits)
+    return bits.view(torch.float64).to(torch.float32)
+
+
+def swiglu_backward(
+    x: QuantTensor,
+    grad_out: torch.Tensor,
+    weight: torch.Tensor,
+    pos_to_token_topk: torch.Tensor,
+    token_topk_to_pos: torch.Tensor,
+    num_per_channels: int,
+    swiglu_clamp_value: Optional[float] = None,
+):
+    """Backward of ``out = silu(g) * u * w`` on the dequantised forward input, in fp32.
+
+    Same arguments and results as ``tile_kernels.torch.swiglu_backward``
+    (tile_kernels/torch/swiglu.py:98-227): ``(out, x_grad_full, weight_grad)`` with
+    ``x_grad_full = [d/dgate | d/dup]``.  Every product below is one fp32 rounding, in the
+    reference's order; the only fused operation is ``fma(g, 1 - s, 1)``.
+    """
+    codes, sf = x
+    assert num_per_channels in (32, 128)
+    assert codes.dtype == torch.float8_e4m3fn and codes.is_contiguous()
+    assert sf.dim() == 2 and sf.is_contiguous() and sf.dtype == torch.float32
+    assert weight.dim() == 2 and weight.is_contiguous()
+    assert pos_to_token_topk.dim() == 1
+    assert token_topk_to_pos.dim() == 2 and token_topk_to_pos.is_contiguous()
+    assert codes.size(-1) % (2 * num_per_channels) == 0
+    hid = codes.size(-1) // 2
+    codes = codes.view(-1, 2 * hid)
+    grad_out = grad_out.view(-1, hid)
+    rows = codes.size(0)
+    num_tokens, num_topk = token_topk_to_pos.shape
+    assert sf.shape == (rows, 2 * hid // num_per_channels)
+    assert grad_out.shape == (rows, hid)
+    assert weight.shape == (num_tokens, num_topk)
+    assert pos_to_token_topk.shape == (rows,)
+
+    xf = codes.to(torch.float32) * sf.repeat_interleave(num_per_channels, dim=1)
+    gate, up = xf[:, :hid].clone(), xf[:, hid:].clone()
+
+    gate_clamped = up_clamped = None
+    if swiglu_clamp_value is not None:
+        c = swiglu_clamp_value
+        gate_clamped = gate > c
+        up_hi, up_lo = up > c, up < -c
+        up_clamped = up_hi | up_lo
+        gate[gate_clamped] = c
+        up[up_hi] = c
+        up[up_lo] = -c
+
+    denom = 1.0 + torch.exp(-gate)
+    sig = torch.ones_like(gate) / denom
+
+    live = pos_to_token_topk >= 0
+    idx = pos_to_token_topk[live].long()
+    w = torch.zeros(rows, dtype=torch.float32)
+    w[live] = weight.reshape(-1).to(torch.float32)[idx]
+
+    go = grad_out.to(torch.float32)
+    go_ws = go * w[:, None] * sig
+    gate_grad = go_ws * up * fma_f32(gate, 1.0 - sig, torch.ones((), dtype=torch.float32))
+    up_grad = go_ws * gate
+    if swiglu_clamp_value is not None:
+        gate_grad[gate_clamped] = 0.0
+        up_grad[up_clamped] = 0.0
+
+    act = gate / denom * up
+    out = act * w[:, None]
+
+    weight_grad = torch.zeros_like(weight)
+    dots = (go * act).sum(dim=1)
+    weight_grad.view(-1)[idx] = dots[live]
+    return out, torch.cat([gate_grad, up_grad], dim=1), weight_grad
+
+
+def swiglu_backward_and_per_token_cast(
+    x: QuantTensor,
+    grad_out: torch.Tensor,
+    weight: torch.Tensor,
+    pos_to_token_topk: torch.Tensor,
+    token_topk_to_pos: torch.Tensor,
+    num_per_channels: int,
+    round_sf: bool = False,
+    swiglu_clamp_value: Optional[float] = None,
+):
+    """Composition the reference's own test uses as ground truth for the fused backward op
+    (tests/quant/test_swiglu_backward_and_per_token_cast.py:78-97): fp32 backward, per-token
+    1 x N E4M3 cast of the fp32 input gradient, and bf16 roundings of the output and the gradient.
+
+    Returns ``(out_bf16, (x_grad_codes, x_grad_sf), x_grad_bf16, weight_grad)``.
+    """
+    out, x_grad, weight_grad = swiglu_backward(x, grad_out, weight, pos_to_token_topk, token_topk_to_pos,
+                                               num_per_channels, swiglu_clamp_value)
+    q = cast(x_grad, 'e4m3', (1, num_per_channels), round_sf=round_sf)
+    return out.to(grad_out.dtype), q, x_grad.to(grad_out.dtype), weight_grad
 
 
 # --------------------------------------------------------------------------------------------------

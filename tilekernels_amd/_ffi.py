@@ -38,6 +38,10 @@ SIGNATURES = {
     'tk_check_get_fused_mapping': (_i32, [_vp, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64]),
     'tk_expand_to_fused': (_i32, [_vp, _i64, _i64, _vp, _i32, _vp, _i64, _vp, _vp, _i32, _vp, _i64, _i32, _vp]),
     'tk_check_expand_to_fused': (_i32, [_vp, _i64, _i64, _vp, _i32, _vp, _i64, _vp, _vp, _i32, _vp, _i64, _i32]),
+    'tk_swiglu_backward_per_token_cast': (_i32, [_vp, _vp, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp,
+                                                 _i32, _i32, _f32, _vp]),
+    'tk_check_swiglu_backward_per_token_cast': (_i32, [_vp, _vp, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp,
+                                                       _vp, _i32, _i32, _f32]),
     'tk_strerror': (ctypes.c_char_p, [_i32]),
     'tk_version': (_i32, []),
 }

@@ -9,6 +9,7 @@
 //
 // Reference semantics: tile_kernels/quant/swiglu_forward_and_per_token_cast_kernel.py:61-170,
 // tile_kernels/torch/swiglu.py:62-86.
+#include "swiglu_math.hpp"
 #include "tk_device.hpp"
 #include "tk_host.hpp"
 
@@ -49,57 +50,6 @@ struct SwigluParams {
     (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).R, (p).H, (p).tiles_m, (p).tiles_k, (p).floor_, (p).clamp,       \
         (p).round_sf, (p).sf.layout, (p).pos_to_expert, (p).pos_to_token_topk, (p).topk_weights, (p).clamped_count, \
         (p).num_weights, (p).sf.nk
-
-// silu(g) * u = g / (1 + exp(-g)) * u in fp32, built on v_exp_f32 / v_rcp_f32 (about 1 ulp each).
-// The reference's CPU evaluation (vectorised exp, IEEE division) is itself only faithful to about
-// 1 ulp in exp, so bit equality is not defined for this op; what can be matched is everything after
-// the exp: 1 + e is one IEEE addition, the quotient is corrected to (almost always) the IEEE
-// quotient, and the two products are single roundings in the reference's order.
-//
-// exp(-g) = 2^(g * -log2 e).  Rounding that product would put |g|*2^-24 of absolute error into the
-// exponent, so the constant is split into hi + lo and the lo part is applied to first order:
-// 2^(g*hi + g*lo) = 2^(g*hi) * (1 + g*lo*ln 2).
-//   bf16 input: hi keeps 15 significant bits, so g*hi is exact for an 8-bit significand
-//   fp32 input: the rounding error of g*hi is recovered with an fma and joins the lo term
-// The gate is capped at -88 inside the exponential only (the CPU's exp overflows to inf at -88.7 and
-// its quotient becomes -0): e and d then stay finite, the reciprocal underflows and the corrected
-// quotient is -0 or a value below 1e-36, never inf * 0.
-#ifndef TK_SWIGLU_NEWTON
-#define TK_SWIGLU_NEWTON 1
-#endif
-
-// g / d from r ~ 1/d: one Newton step on the quotient (two fmas)
-__device__ __forceinline__ float quotient(float g, float d) {
-    const float r = __builtin_amdgcn_rcpf(d);
-    const float q0 = g * r;
-#if TK_SWIGLU_NEWTON
-    return __builtin_fmaf(__builtin_fmaf(-d, q0, g), r, q0);
-#else
-    return q0;
-#endif
-}
-
-template <typename InT> __device__ __forceinline__ float silu_mul(float g, float u);
-
-template <> __device__ __forceinline__ float silu_mul<bf16_t>(float g, float u) {
-    constexpr float nh = -1.44268798828125f;             // -log2(e) cut to 15 significant bits (0xBFB8AA00)
-    constexpr float nl_ln2 = -4.8884952e-06f;            // (-log2(e) - nh) * ln 2
-    const float gc = __builtin_fmaxf(g, -88.0f);
-    const float e0 = __builtin_amdgcn_exp2f(gc * nh);    // exact product
-    const float e = __builtin_fmaf(e0, gc * nl_ln2, e0);
-    return quotient(g, 1.0f + e) * u;
-}
-
-template <> __device__ __forceinline__ float silu_mul<float>(float g, float u) {
-    constexpr float nh = -1.4426950216293335f;           // float(-log2 e)
-    constexpr float nl = -1.9259629911266175e-8f;        // -log2 e - nh
-    const float gc = __builtin_fmaxf(g, -88.0f);
-    const float th = gc * nh;
-    const float tl = __builtin_fmaf(gc, nl, __builtin_fmaf(gc, nh, -th));
-    const float e0 = __builtin_amdgcn_exp2f(th);
-    const float e = __builtin_fmaf(e0, tl * 0.6931471805599453f, e0);
-    return quotient(g, 1.0f + e) * u;
-}
 
 // CLAMP: 0 none, 1 clamp, 2 clamp and count
 template <int CLAMP> struct ClampCounter {
