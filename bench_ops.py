@@ -1,0 +1,213 @@
+#!/usr/bin/env python3
+"""Kernel timings of the operators around the headline path, one JSON line per operator.
+
+    python bench_ops.py [--steps 2000] [--warmup 1000] [--only NAME]
+
+Companion of bench.py (which measures the headline workload and keeps the driver's contract): the
+same method -- C-ABI calls on preallocated device buffers, buffer sets rotated past the 256 MB
+last-level cache, HIP events on the launch stream over the timed region -- applied to the
+dequantisation, the re-quantisation of quantised input, the MoE layout helpers and the fused SwiGLU
+backward.  `bytes` is the algorithmic HBM traffic of one call (inputs read once, outputs written
+once); `frac` prices it against 8 TB/s.
+"""
+import argparse
+import json
+import os
+import sys
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+LLC_BYTES = 256 << 20
+
+
+def nbytes(*tensors) -> int:
+    return sum(t.numel() * t.element_size() for t in tensors)
+
+
+class Op:
+    """`build()` returns (callable launching one call on torch's current stream, algorithmic bytes,
+    footprint bytes of the buffer set)."""
+
+    def __init__(self, name, workload, build):
+        self.name, self.workload, self.build = name, workload, build
+
+
+def _sets_needed(footprint: int) -> int:
+    return max(3, -(-int(1.6 * LLC_BYTES) // max(footprint, 1)))
+
+
+def op_cast_back():
+    import tilekernels_amd as tk
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    M, K = 8192, 4096
+    x = torch.randn((M, K), device='cuda', dtype=torch.bfloat16)
+    codes, sf = tk.quant.per_token_cast(x, 'e4m3', num_per_channels=128)
+    out = torch.empty((M, K), device='cuda', dtype=torch.bfloat16)
+    stream = _ffi.current_stream(x.device)
+
+    def launch():
+        rc = lib.tk_cast_back(codes.data_ptr(), 0, M, K, sf.data_ptr(), sf.stride(0), 0, 1, 128, out.data_ptr(), 0, stream)
+        assert rc == 0, rc
+    return launch, nbytes(codes, sf, out), nbytes(codes, sf, out)
+
+
+def op_requant():
+    import tilekernels_amd as tk
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    M, K = 8192, 4096
+    x = torch.randn((M, K), device='cuda', dtype=torch.bfloat16)
+    codes, sf = tk.quant.per_token_cast(x, 'e4m3', num_per_channels=128)
+    out = torch.empty((M, K // 2), device='cuda', dtype=torch.int8)
+    out_sf = torch.empty((M, K // 32), device='cuda', dtype=torch.float32)
+    stream = _ffi.current_stream(x.device)
+
+    def launch():
+        # E4M3 1x128 -> E2M1 1x32 (the path per_token_cast takes when handed a (codes, scales) pair)
+        rc = lib.tk_per_token_cast_quantized(codes.data_ptr(), 0, M, K, K, sf.data_ptr(), sf.stride(0), 0, 1, 128,
+                                             out.data_ptr(), out_sf.data_ptr(), out_sf.stride(0), 1, 32, 0, 0, stream)
+        assert rc == 0, rc
+    return launch, nbytes(codes, sf, out, out_sf), nbytes(codes, sf, out, out_sf)
+
+
+def _moe_maps(T=4096, K=8, E=256, alignment=128, seed=0):
+    import tilekernels_amd as tk
+    g = torch.Generator().manual_seed(seed)
+    topk_idx = torch.topk(torch.rand((T, E), generator=g), K, dim=-1).indices.contiguous().cuda()
+    maps = tk.moe.get_fused_mapping(topk_idx, E, 0, alignment)
+    return topk_idx, maps
+
+
+def op_get_fused_mapping():
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    T, K, E, alignment = 4096, 8, 256, 128
+    topk_idx, maps = _moe_maps(T, K, E, alignment)
+    p2e, p2t, ptt, t2p, es, ee, npe = maps[:7]
+    R = p2e.numel()
+    ws_bytes = lib.tk_fused_mapping_workspace_bytes(T, K, E)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device='cuda')
+    stream = _ffi.current_stream(topk_idx.device)
+
+    def launch():
+        rc = lib.tk_get_fused_mapping(topk_idx.data_ptr(), T, K, E, alignment, R, p2e.data_ptr(), p2t.data_ptr(),
+                                      ptt.data_ptr(), t2p.data_ptr(), es.data_ptr(), ee.data_ptr(), npe.data_ptr(),
+                                      ws.data_ptr(), ws_bytes, stream)
+        assert rc == 0, rc
+    b = nbytes(topk_idx, p2e, p2t, ptt, t2p, es, ee, npe)
+    return launch, b, b
+
+
+def op_expand_to_fused():
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    T, K, hidden = 4096, 8, 4096
+    _, maps = _moe_maps(T, K)
+    p2e, t2p = maps[0], maps[3]
+    R = p2e.numel()
+    x = torch.randn((T, hidden), device='cuda', dtype=torch.bfloat16)
+    out = torch.empty((R, hidden), device='cuda', dtype=torch.bfloat16)
+    stream = _ffi.current_stream(x.device)
+
+    def launch():
+        rc = lib.tk_expand_to_fused(x.data_ptr(), T, hidden * 2, t2p.data_ptr(), K, p2e.data_ptr(), R, out.data_ptr(),
+                                    0, 0, 0, 0, 0, stream)
+        assert rc == 0, rc
+    return launch, nbytes(x, out, t2p, p2e), nbytes(x, out, t2p, p2e)
+
+
+def op_swiglu_backward(group=128, rows=8192, hidden=2048):
+    def build():
+        import tilekernels_amd as tk
+        from tilekernels_amd import _ffi
+        lib = _ffi.load()
+        R, H, T, K = rows, hidden, rows // 8, 8
+        x = torch.randn((R, 2 * H), device='cuda', dtype=torch.bfloat16)
+        codes, sf = tk.quant.per_token_cast(x, 'e4m3', num_per_channels=group)
+        del x
+        go = torch.randn((R, H), device='cuda', dtype=torch.bfloat16)
+        w = torch.rand((T, K), device='cuda')
+        ptt = torch.randperm(T * K, device='cuda').to(torch.int32)
+        t2p = torch.empty((T * K,), dtype=torch.int32, device='cuda')
+        t2p[ptt.long()] = torch.arange(R, dtype=torch.int32, device='cuda')
+        out = torch.empty((R, H), device='cuda', dtype=torch.bfloat16)
+        q = torch.empty((R, 2 * H), device='cuda', dtype=torch.float8_e4m3fn)
+        q_sf = torch.empty((R, 2 * H // group), device='cuda', dtype=torch.float32)
+        xg = torch.empty((R, 2 * H), device='cuda', dtype=torch.bfloat16)
+        wg = torch.empty((T, K), device='cuda')
+        stream = _ffi.current_stream(go.device)
+
+        def launch():
+            rc = lib.tk_swiglu_backward_per_token_cast(codes.data_ptr(), sf.data_ptr(), R, H, group, go.data_ptr(),
+                                                       w.data_ptr(), ptt.data_ptr(), t2p.data_ptr(), T * K, out.data_ptr(),
+                                                       q.data_ptr(), q_sf.data_ptr(), xg.data_ptr(), wg.data_ptr(), 1, 0, 0.0,
+                                                       stream)
+            assert rc == 0, rc
+        b = nbytes(codes, sf, go, w, ptt, t2p, out, q, q_sf, xg, wg)
+        return launch, b, b
+    return build
+
+
+OPS = [
+    Op('cast_back', 'cast_back e4m3 1x128 -> bf16, [8192,4096]', op_cast_back),
+    Op('per_token_cast_quantized', 'per_token_cast of (e4m3 1x128) input -> e2m1 1x32, [8192,4096]', op_requant),
+    Op('get_fused_mapping', 'get_fused_mapping 4096 tokens, top-8 of 256 experts, pad 128', op_get_fused_mapping),
+    Op('expand_to_fused', 'expand_to_fused bf16 [4096,4096] -> [R,4096], top-8 of 256 experts, pad 128', op_expand_to_fused),
+    Op('swiglu_backward_and_per_token_cast', 'swiglu_backward_and_per_token_cast 1x128 round_sf, x e4m3 [8192,4096]',
+       op_swiglu_backward(128)),
+    Op('swiglu_backward_and_per_token_cast_g32', 'swiglu_backward_and_per_token_cast 1x32 round_sf, x e4m3 [8192,4096]',
+       op_swiglu_backward(32)),
+]
+
+
+def run(op: Op, steps: int, warmup: int) -> dict:
+    sets = []
+    launch, algo, footprint = op.build()
+    sets.append(launch)
+    for _ in range(_sets_needed(footprint) - 1):
+        sets.append(op.build()[0])
+    n = len(sets)
+    for i in range(warmup):
+        sets[i % n]()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        sets[i % n]()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / steps
+    gbs = algo / us / 1e3
+    return {'op': op.name, 'workload': op.workload, 'us_per_call': round(us, 2), 'bytes': algo, 'GB/s': round(gbs, 1),
+            'frac': round(gbs / HBM_PEAK_GBS, 4), 'buffer_sets': n, 'steps': steps, 'warmup': warmup}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--steps', type=int, default=2000)
+    ap.add_argument('--warmup', type=int, default=1000)
+    ap.add_argument('--only', type=str, default=None)
+    ap.add_argument('--copy-calibration', action='store_true',
+                    help='also run plain 256 MiB device copies (reference point for hardware-counter runs)')
+    a = ap.parse_args()
+    if not torch.cuda.is_available():
+        sys.exit('bench_ops.py needs a GPU')
+    torch.cuda.set_device(0)
+    for op in OPS:
+        if a.only and a.only != op.name:
+            continue
+        print(json.dumps(run(op, a.steps, a.warmup)), flush=True)
+        torch.cuda.empty_cache()
+    if a.copy_calibration:
+        from bench import copy_calibration
+        print(json.dumps(copy_calibration()), flush=True)
+
+
+if __name__ == '__main__':
+    main()

@@ -2,8 +2,8 @@
 //
 // out[m, k] = float(code[m, k]) * sf[m / bm, k / bk], one fp32 product, then (for bf16) one
 // round-to-nearest-even conversion (v_cvt_pk_bf16_f32).  Pure streaming: a lane takes 8 consecutive
-// codes (8 or 4 bytes), their shared scale, and writes 16 (bf16) or 32 (fp32) bytes; a workgroup of
-// 4 waves covers 8 rows x 512 columns.
+// codes (8 or 4 bytes), their shared scale, and writes 16 (bf16) or 32 (fp32) bytes; a workgroup
+// covers 2 rows x up to 4096 columns (row-major scales) or 8 rows x 512 columns.
 //
 // Reference semantics: tile_kernels/quant/cast_back_kernel.py:19-75 (kernel) and :77-143 (wrappers),
 // tile_kernels/torch/cast.py:40-59 (oracle).
@@ -16,16 +16,21 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kBackRowsPerWave = 2;
 
-template <typename InT, bool OUT_F32, bool FULL>
-__global__ __launch_bounds__(kThreads) void cast_back_kernel(const void *x, void *out, void *a_sf, int64_t a_sf_ld, int M, int K,
-                                                             int tiles_k, int a_sf_layout, int nm, int nk, int bm, int bk) {
-    constexpr int RPW = kBackRowsPerWave, ROWS = kWaves * RPW;
+// WIDE: the workgroup's waves stand side by side on the same RPW rows (row-major scales: one
+// workgroup then reads a row's scales once, instead of eight workgroups on eight L2s each fetching
+// the line for 16 bytes of it); otherwise the 4 waves are stacked, 512 columns wide.
+template <typename InT, bool OUT_F32, bool WIDE, bool FULL>
+__global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_back_kernel(const void *x, void *out, void *a_sf, int64_t a_sf_ld,
+                                                                                         int M, int K, int tiles_k, int a_sf_layout, int nm,
+                                                                                         int nk, int bm, int bk) {
+    constexpr int RPW = kBackRowsPerWave, ROWS = WIDE ? RPW : kWaves * RPW;
     const SfRef sf{a_sf, a_sf_ld, a_sf_layout, nm, nk};
     const int tile_m = blockIdx.x / tiles_k, tile_k = blockIdx.x - tile_m * tiles_k;
     const int lane = threadIdx.x & 63, wave = wave_id();
-    const int col = tile_k * kStripCols + lane * 8;
+    const int strip = WIDE ? tile_k * (int)(blockDim.x >> 6) + wave : tile_k;
+    const int col = strip * kStripCols + lane * 8;
     const bool col_ok = FULL || col < K;
-    const int row0 = tile_m * ROWS + wave * RPW;
+    const int row0 = tile_m * ROWS + (WIDE ? 0 : wave * RPW);
 
     Raw8<InT> raw[RPW];
 #pragma unroll
@@ -55,18 +60,28 @@ __global__ __launch_bounds__(kThreads) void cast_back_kernel(const void *x, void
     }
 }
 
+template <typename InT, bool OUT_F32, bool WIDE>
+static void launch_cast_back_2(const void *x, void *out, const void *sf, int64_t sf_ld, int M, int K, int sf_layout, int bm, int bk,
+                               hipStream_t stream) {
+    const int strips = (K + kStripCols - 1) / kStripCols;
+    const int waves = WIDE ? wide_tile_waves(strips) : kWaves;
+    const int rows = WIDE ? kBackRowsPerWave : kWaves * kBackRowsPerWave;
+    const int cols = WIDE ? waves * kStripCols : kStripCols;
+    const int tiles_m = (M + rows - 1) / rows, tiles_k = (K + cols - 1) / cols;
+    const int nm = (M + bm - 1) / bm, nk = (K + bk - 1) / bk;
+    const dim3 grid((unsigned)(tiles_m * tiles_k)), block(64 * waves);
+    void *sfp = const_cast<void *>(sf);
+    if (M % rows == 0 && K % cols == 0)
+        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, true>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, tiles_k, sf_layout, nm, nk, bm, bk);
+    else
+        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, false>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, tiles_k, sf_layout, nm, nk, bm, bk);
+}
+
 template <typename InT, bool OUT_F32>
 static hipError_t launch_cast_back(const void *x, void *out, const void *sf, int64_t sf_ld, int M, int K, int sf_layout,
                                    int bm, int bk, hipStream_t stream) {
-    constexpr int ROWS = kWaves * kBackRowsPerWave;
-    const int tiles_m = (M + ROWS - 1) / ROWS, tiles_k = (K + kStripCols - 1) / kStripCols;
-    const int nm = (M + bm - 1) / bm, nk = (K + bk - 1) / bk;
-    const dim3 grid((unsigned)(tiles_m * tiles_k)), block(kThreads);
-    void *sfp = const_cast<void *>(sf);
-    if (M % ROWS == 0 && K % kStripCols == 0)
-        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, true>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, tiles_k, sf_layout, nm, nk, bm, bk);
-    else
-        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, false>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, tiles_k, sf_layout, nm, nk, bm, bk);
+    if (sf_layout == TK_SF_ROW_F32) launch_cast_back_2<InT, OUT_F32, true>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);
+    else launch_cast_back_2<InT, OUT_F32, false>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);
     return hipGetLastError();
 }
 
@@ -89,7 +104,7 @@ extern "C" int tk_check_cast_back(const void *x, int x_fmt, int64_t M, int64_t K
     const int64_t nm = (M + bm - 1) / bm, nk = (K + bk - 1) / bk;
     const int64_t need = x_sf_layout == TK_SF_ROW_F32 ? nk : (x_sf_layout == TK_SF_COL_F32 ? nm : 4 * nm);
     if (x_sf_ld < need) return TK_ERR_BAD_STRIDE;
-    if (((M + 7) / 8) * ((K + kStripCols - 1) / kStripCols) > INT32_MAX) return TK_ERR_TOO_LARGE;
+    if (((M + 1) / 2) * ((K + kStripCols - 1) / kStripCols) > INT32_MAX - 8) return TK_ERR_TOO_LARGE;
     return TK_OK;
 }
 

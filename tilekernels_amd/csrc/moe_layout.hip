@@ -47,34 +47,61 @@ __global__ __launch_bounds__(kThreads) void fused_mapping_count_kernel(const int
         for (int e = lane; e < num_experts; e += 64) ws[(int64_t)slice * num_experts + e] = h[e];
 }
 
+// One workgroup of 1024 threads.  The slice axis is cut into C = 1024 / num_experts chunks (at least
+// one) and thread (c, e) owns chunk c of expert e: it sums its chunk (independent loads, so their
+// latencies overlap), the chunk totals are exchanged through LDS, and a second walk over the chunk
+// (from L2) writes the exclusive offsets.  Expert starts come from a block-wide prefix sum.
 __global__ __launch_bounds__(1024) void fused_mapping_scan_kernel(int32_t *ws, int num_slices, int num_experts, int alignment,
                                                                   int32_t *expert_start, int32_t *expert_end,
                                                                   int32_t *num_tokens_per_expert) {
+    __shared__ int32_t total[1024];          // [chunk][expert], chunks * num_experts <= 1024
     __shared__ int32_t padded[kMaxExperts];
-    __shared__ int32_t start[kMaxExperts];
-    for (int e = threadIdx.x; e < num_experts; e += blockDim.x) {
-        int32_t run = 0;
-        for (int s = 0; s < num_slices; ++s) {
+    __shared__ int32_t scan[2][kMaxExperts];
+    const int chunks = num_experts >= 1024 ? 1 : 1024 / num_experts;
+    const int per = (num_slices + chunks - 1) / chunks;
+    const int c = threadIdx.x / num_experts, e = threadIdx.x - c * num_experts;
+    const bool active = c < chunks;
+    const int s0 = c * per, s1 = min(s0 + per, num_slices);
+
+    if (active) {
+        int32_t sum = 0;
+#pragma unroll 8
+        for (int s = s0; s < s1; ++s) sum += ws[(int64_t)s * num_experts + e];
+        total[c * num_experts + e] = sum;
+    }
+    __syncthreads();
+    int32_t run = 0;
+    if (active) {
+        for (int k = 0; k < c; ++k) run += total[k * num_experts + e];
+        if (c == 0) {
+            int32_t all = 0;
+            for (int k = 0; k < chunks; ++k) all += total[k * num_experts + e];
+            padded[e] = (all + alignment - 1) / alignment * alignment;
+        }
+#pragma unroll 8
+        for (int s = s0; s < s1; ++s) {
             const int64_t at = (int64_t)s * num_experts + e;
-            const int32_t c = ws[at];
+            const int32_t n = ws[at];
             ws[at] = run;          // exclusive offset of this slice inside the expert
-            run += c;
-        }
-        padded[e] = (run + alignment - 1) / alignment * alignment;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int32_t run = 0;
-        for (int e = 0; e < num_experts; ++e) {
-            start[e] = run;
-            run += padded[e];
+            run += n;
         }
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < num_experts; e += blockDim.x) {
-        expert_start[e] = start[e];
-        expert_end[e] = start[e] + padded[e];
-        num_tokens_per_expert[e] = padded[e];
+    // inclusive prefix sum of padded[] over the experts (Hillis-Steele, ping-pong buffers)
+    const int t = threadIdx.x;
+    scan[0][t] = t < num_experts ? padded[t] : 0;
+    __syncthreads();
+    int cur = 0;
+    for (int d = 1; d < kMaxExperts; d <<= 1) {
+        scan[cur ^ 1][t] = scan[cur][t] + (t >= d ? scan[cur][t - d] : 0);
+        cur ^= 1;
+        __syncthreads();
+    }
+    if (t < num_experts) {
+        const int32_t end = scan[cur][t];
+        expert_start[t] = end - padded[t];
+        expert_end[t] = end;
+        num_tokens_per_expert[t] = padded[t];
     }
 }
 
@@ -125,9 +152,12 @@ __global__ __launch_bounds__(kThreads) void fused_mapping_assign_kernel(const in
 
 // ------------------------------------------------------------------------------------------------
 // expand_to_fused: workgroup t < T copies row t to each of its positions (read once, written once
-// per destination); workgroup T + r zero-fills row r when it is padding.  Rows are moved as raw
+// per destination); the workgroups after those walk the expanded rows, 4 per wave, and zero-fill
+// the ones that are padding.  Rows are moved as raw
 // 16-byte pieces, so any element type works.  Optional 4-byte scale rows travel the same way into a
 // row-major or column-major scale tensor.
+constexpr int kPadRowsPerWave = 4;
+
 __global__ __launch_bounds__(kThreads) void expand_to_fused_kernel(const uint8_t *x, int64_t row_bytes, const int32_t *token_topk_to_pos,
                                                                    int num_topk, const int32_t *pos_to_expert, int num_tokens,
                                                                    int num_expanded, uint8_t *out, const uint32_t *x_sf, int sf_cols,
@@ -154,13 +184,17 @@ __global__ __launch_bounds__(kThreads) void expand_to_fused_kernel(const uint8_t
             }
         }
     } else {
-        const int r = b - num_tokens;
-        if (uniform_load(pos_to_expert + r) >= 0) return;
-        uint8_t *dst = out + (int64_t)r * row_bytes;
-        for (int64_t off = (int64_t)threadIdx.x * 16; off < row_bytes; off += kThreads * 16)
-            __builtin_nontemporal_store(u32x4{0u, 0u, 0u, 0u}, reinterpret_cast<u32x4 *>(dst + off));
-        if (x_sf)
-            for (int j = threadIdx.x; j < sf_cols; j += kThreads) out_sf[sf_col_major ? (int64_t)j * out_sf_ld + r : (int64_t)r * out_sf_ld + j] = 0u;
+        // a wave looks at kPadRowsPerWave consecutive rows and clears the ones that are padding
+        const int lane = threadIdx.x & 63;
+        const int first = ((b - num_tokens) * kWaves + wave_id()) * kPadRowsPerWave;
+        for (int r = first; r < first + kPadRowsPerWave && r < num_expanded; ++r) {
+            if (uniform_load(pos_to_expert + r) >= 0) continue;
+            uint8_t *dst = out + (int64_t)r * row_bytes;
+            for (int64_t off = (int64_t)lane * 16; off < row_bytes; off += 64 * 16)
+                __builtin_nontemporal_store(u32x4{0u, 0u, 0u, 0u}, reinterpret_cast<u32x4 *>(dst + off));
+            if (x_sf)
+                for (int j = lane; j < sf_cols; j += 64) out_sf[sf_col_major ? (int64_t)j * out_sf_ld + r : (int64_t)r * out_sf_ld + j] = 0u;
+        }
     }
 }
 
@@ -250,7 +284,8 @@ extern "C" int tk_expand_to_fused(const void *x, int64_t num_tokens, int64_t row
     const int rc = tk_check_expand_to_fused(x, num_tokens, row_bytes, token_topk_to_pos, num_topk, pos_to_expert, num_expanded, out,
                                             x_sf, sf_cols, out_sf, out_sf_ld, sf_col_major);
     if (rc != TK_OK) return rc;
-    const int64_t grid = num_tokens + num_expanded;
+    const int64_t rows_per_block = kWaves * kPadRowsPerWave;
+    const int64_t grid = num_tokens + (num_expanded + rows_per_block - 1) / rows_per_block;
     if (grid == 0) return TK_OK;
     hipLaunchKernelGGL(expand_to_fused_kernel, dim3((unsigned)grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint8_t *>(x), row_bytes, token_topk_to_pos, num_topk, pos_to_expert, (int)num_tokens,
