@@ -158,6 +158,11 @@ __global__ __launch_bounds__(kThreads) void fused_mapping_assign_kernel(const in
 // row-major or column-major scale tensor.
 constexpr int kPadRowsPerWave = 4;
 
+// Non-temporal 16-byte stores.  Measured on MI355X for bf16 [4096, 4096] expanded 8-fold with
+// 128-row padding (394 MB written): 82 us, against 84 us with plain stores; pairs of 8-byte
+// system-scope stores take 320 us.
+__device__ __forceinline__ void expand_store16(void *p, u32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p)); }
+
 __global__ __launch_bounds__(kThreads) void expand_to_fused_kernel(const uint8_t *x, int64_t row_bytes, const int32_t *token_topk_to_pos,
                                                                    int num_topk, const int32_t *pos_to_expert, int num_tokens,
                                                                    int num_expanded, uint8_t *out, const uint32_t *x_sf, int sf_cols,
@@ -170,8 +175,7 @@ __global__ __launch_bounds__(kThreads) void expand_to_fused_kernel(const uint8_t
             const u32x4 v = ld_stream16(src + off);
             for (int k = 0; k < num_topk; ++k) {
                 const int p = uniform_load(pos + k);
-                if (p >= 0 && p < num_expanded)
-                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(out + (int64_t)p * row_bytes + off));
+                if (p >= 0 && p < num_expanded) expand_store16(out + (int64_t)p * row_bytes + off, v);
             }
         }
         if (x_sf) {
@@ -191,7 +195,7 @@ __global__ __launch_bounds__(kThreads) void expand_to_fused_kernel(const uint8_t
             if (uniform_load(pos_to_expert + r) >= 0) continue;
             uint8_t *dst = out + (int64_t)r * row_bytes;
             for (int64_t off = (int64_t)lane * 16; off < row_bytes; off += 64 * 16)
-                __builtin_nontemporal_store(u32x4{0u, 0u, 0u, 0u}, reinterpret_cast<u32x4 *>(dst + off));
+                expand_store16(dst + off, u32x4{0u, 0u, 0u, 0u});
             if (x_sf)
                 for (int j = lane; j < sf_cols; j += 64) out_sf[sf_col_major ? (int64_t)j * out_sf_ld + r : (int64_t)r * out_sf_ld + j] = 0u;
         }

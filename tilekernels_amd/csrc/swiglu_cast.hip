@@ -243,7 +243,10 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KER
 
 // Rows per wave of the tiled kernel.  Measured on MI355X at [8192, 4096] bf16 (us per call, row-major
 // scales): 1 row 16.5, 2 rows 15.7, 4 rows 15.0.
-constexpr int kSwigluRowsPerWave = 4;
+#ifndef TK_SWIGLU_RPW
+#define TK_SWIGLU_RPW 4
+#endif
+constexpr int kSwigluRowsPerWave = TK_SWIGLU_RPW;
 
 template <typename InT, int CLAMP, int RPW, bool WIDE>
 static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t stream) {
