@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define TK_QUANT_VERSION 104 /* major*10000 + minor*100 + patch */
+#define TK_QUANT_VERSION 105 /* major*10000 + minor*100 + patch */
 
 enum tk_dtype { TK_BF16 = 0, TK_F32 = 1 };
 enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1 };
@@ -172,6 +172,31 @@ int tk_check_swiglu_backward_per_token_cast(const void *x, const float *x_sf, in
                                             int64_t num_weights, const void *out, const void *x_grad_codes,
                                             const float *x_grad_sf, const void *x_grad, const float *weight_grad,
                                             int round_sf, int use_clamp, float clamp);
+
+/*
+ * Per-channel cast: E4M3 with one scale per `num_per_tokens` (32 or 128) tokens x 1 column, scales fp32
+ * row-major out_sf[ceil(M / num_per_tokens), K].  The input is
+ *   x_sf == NULL, swiglu == 0 : bf16 x[num_tokens, K]
+ *   x_sf != NULL              : E4M3 codes x[num_tokens, K] with fp32 scales x_sf[num_tokens, K / 128]
+ *                               (1 x 128 groups); every element is first dequantised, code * scale
+ *   swiglu != 0               : bf16 x[num_tokens, 2K]; the value cast is bf16(g / (1 + exp(-g)) * u) with
+ *                               g = x[:, :K], u = x[:, K:], clamped as in tk_swiglu_per_token_cast with use_clamp
+ * pos_to_token (NULL, or int32[M]) gathers rows: output row r comes from input row pos_to_token[r], a
+ * negative index gives a row of zeros; without it M rows are taken in order (num_tokens >= M).
+ * transpose == 0: out[M, K];  transpose != 0: out[K, M].
+ * Stands behind tile_kernels.quant.per_channel_cast, per_channel_cast_fused
+ * (tile_kernels/quant/per_channel_cast_fused_kernel.py:130-203), per_channel_cast_and_transpose
+ * (per_channel_cast_and_transpose_kernel.py:84-123) and swiglu_forward_and_per_channel_cast_and_transpose
+ * (swiglu_forward_and_per_channel_cast_and_transpose_kernel.py:178-231).
+ *   requirements K % 8 == 0 (K % 128 == 0 with x_sf); M % 16 == 0; x 16-byte (codes: 8-byte) aligned;
+ *                out 8-byte, transposed 16-byte aligned
+ */
+int tk_per_channel_cast(const void *x, int x_dtype, const float *x_sf, int64_t num_tokens, int64_t K,
+                        const int32_t *pos_to_token, int64_t M, void *out, float *out_sf, int num_per_tokens, int round_sf,
+                        int transpose, int swiglu, int use_clamp, float clamp, void *stream);
+int tk_check_per_channel_cast(const void *x, int x_dtype, const float *x_sf, int64_t num_tokens, int64_t K,
+                              const int32_t *pos_to_token, int64_t M, const void *out, const float *out_sf,
+                              int num_per_tokens, int round_sf, int transpose, int swiglu, int use_clamp, float clamp);
 
 /*
  * Dequantisation: out[m, k] = float(code[m, k]) * sf[m / bm, k / bk] (one fp32 product), stored as

@@ -6,6 +6,7 @@ pure-torch implementations:
 * ``cast`` / ``cast_back``      <- tile_kernels/torch/cast.py:62-221 and :40-59
 * ``swiglu_forward``            <- tile_kernels/torch/swiglu.py:9-88
 * ``swiglu_backward``           <- tile_kernels/torch/swiglu.py:90-227
+* ``per_channel_cast_fused``    <- tile_kernels/torch/per_channel_cast_fused.py:9-46
 * ``unpack_from_e2m1fn_x2``     <- tile_kernels/quant/common.py:247-295
 * ``encode_e2m1``               <- tile_kernels/torch/cast.py:224-252 (same result, closed form)
 
@@ -26,6 +27,9 @@ How each function is pinned (all pins live in tests/test_oracle_*.py and run wit
 * the whole of ``cast`` is cross-checked bit-for-bit against the independent scalar C
   restatement in oracle/quant_ref.c.
 * ``swiglu_forward`` is checked against float64 evaluation and ``torch.nn.functional.silu``.
+* ``per_channel_cast_fused`` and the two transposing compositions reduce to ``cast`` with block
+  (N, 1); that geometry is checked against a naive column loop and the C restatement, the gather
+  against hand-built index lists.
 * ``swiglu_backward`` is checked against float64 autograd of ``silu(g) * u * w`` (a dropped term,
   a wrong sign or swapped halves fails it), against hand-set clamp cases, and its ``fma_f32`` helper
   against the C library's correctly rounded ``fmaf`` on operands built to hit double rounding.
@@ -418,6 +422,56 @@ def swiglu_backward_and_per_token_cast(
                                                num_per_channels, swiglu_clamp_value)
     q = cast(x_grad, 'e4m3', (1, num_per_channels), round_sf=round_sf)
     return out.to(grad_out.dtype), q, x_grad.to(grad_out.dtype), weight_grad
+
+
+def per_channel_cast_fused(
+    x: Union[torch.Tensor, QuantTensor],
+    num_per_tokens: int,
+    num_per_channels: Optional[int],
+    round_sf: bool,
+    pos_to_token: Optional[torch.Tensor],
+) -> QuantTensor:
+    """Per-channel cast (one scale per ``num_per_tokens`` tokens of a column) with the optional row
+    gather and the optional dequantisation of an FP8 input with 1 x ``num_per_channels`` scales.
+
+    Same arguments and results as the reference's torch statement
+    (tile_kernels/torch/per_channel_cast_fused.py:9-46): gathered rows with a negative index are
+    zero rows (zero codes and zero scales for a quantised input), then ``cast`` with block
+    ``(num_per_tokens, 1)``.
+    """
+    quantised = isinstance(x, tuple)
+    if pos_to_token is not None:
+        data = x[0] if quantised else x
+        idx = pos_to_token.clamp(min=0).long()
+        live = (pos_to_token >= 0)[:, None]
+        rows = torch.where(live, data[idx].to(torch.float32), torch.zeros((), dtype=torch.float32)).to(data.dtype)
+        if quantised:
+            sf_rows = torch.where(live, x[1][idx], torch.zeros((), dtype=x[1].dtype))
+            x = (rows, sf_rows)
+        else:
+            x = rows
+    return cast(x, 'e4m3', block_size=(num_per_tokens, 1),
+                x_block_size=(1, num_per_channels) if quantised else None, round_sf=round_sf)
+
+
+def per_channel_cast_and_transpose(x: torch.Tensor, num_per_tokens: int, round_sf: bool) -> QuantTensor:
+    """What the reference's test expects of the transposing variant
+    (tests/quant/test_per_channel_cast_and_transpose.py:45-48): the per-channel cast, codes transposed."""
+    codes, sf = cast(x, 'e4m3', block_size=(num_per_tokens, 1), round_sf=round_sf)
+    return codes.T.contiguous(), sf
+
+
+def swiglu_forward_and_per_channel_cast_and_transpose(x: torch.Tensor, num_per_tokens: int, round_sf: bool = False,
+                                                      without_transpose: bool = False,
+                                                      swiglu_clamp_value: Optional[float] = None) -> QuantTensor:
+    """Composition the reference's test uses as ground truth
+    (tests/quant/test_swiglu_forward_and_per_channel_cast_and_transpose.py:62-75): SwiGLU in fp32,
+    rounded to bf16, per-channel cast, codes transposed unless ``without_transpose``."""
+    act = swiglu_forward(x, swiglu_clamp_value=swiglu_clamp_value).to(torch.bfloat16)
+    codes, sf = cast(act, 'e4m3', block_size=(num_per_tokens, 1), round_sf=round_sf)
+    if not without_transpose:
+        codes = codes.T.contiguous()
+    return codes, sf
 
 
 # --------------------------------------------------------------------------------------------------

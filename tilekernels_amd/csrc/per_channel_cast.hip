@@ -1,0 +1,292 @@
+// Per-channel (N tokens x 1 column, N in {32, 128}) E4M3 cast for gfx950, with the fusions the
+// reference offers around it: row gather (pos_to_token), dequantisation of an E4M3 input with 1 x 128
+// scales, SwiGLU in front, and a transposed ([K, M]) output.
+//
+// A workgroup of 8 waves owns a 128-token x 256-column tile and keeps it in registers between the
+// amax and the conversion, so HBM is read once.  Half a wave (32 lanes x 8 columns = 256 columns)
+// takes 8 consecutive tokens: wave w, half h holds tokens 16 w + 8 h + p, p = 0..7.  A lane
+// therefore owns 8 columns over 8 tokens and reduces |x| down its columns without any cross-lane
+// step; the 16 partial maxima per column (8 waves x 2 halves) meet in LDS, thread c < 256 derives
+// the scale(s) of column c (one division per scale in the whole workgroup, stored as one coalesced
+// run) and hands the multipliers back through LDS.
+//   plain output      : a lane converts 8 columns of a token -> one 8-byte store, 256 bytes per half-wave
+//   transposed output : a lane converts 8 tokens of a column -> 8 bytes of an output row; the tile is
+//                       turned in LDS ([256 columns][128 tokens] bytes) and leaves as 128-byte row pieces
+//
+// Reference semantics: tile_kernels/quant/per_channel_cast_fused_kernel.py:16-203,
+// per_channel_cast_and_transpose_kernel.py:8-123,
+// swiglu_forward_and_per_channel_cast_and_transpose_kernel.py:9-231; oracle
+// tile_kernels/torch/per_channel_cast_fused.py and tile_kernels/torch/cast.py with block (N, 1).
+#include "swiglu_math.hpp"
+#include "tk_device.hpp"
+#include "tk_host.hpp"
+
+namespace tk {
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kPcTileM = 128, kPcTileK = 256, kPcThreads = 512, kPcRows = 8;   // kPcRows tokens per lane
+constexpr int kPcPitch = kPcTileM + 16;                                          // bytes per column in the turned tile
+
+enum { PC_BF16 = 0, PC_E4M3 = 1, PC_SWIGLU = 2 };
+
+struct PerChannelParams {
+    const void *x;
+    const float *x_sf;
+    const int32_t *pos_to_token;
+    uint8_t *out;
+    float *out_sf;
+    int num_tokens, K, M;      // input rows, columns (of the output), output rows
+    int tiles_k;
+    int round_sf, use_clamp;
+    float clamp;
+};
+
+#define TK_PC_KERNEL_ARGS                                                                                          \
+    const void *a_x, uint8_t *a_out, float *a_out_sf, const float *a_x_sf, const int32_t *a_p2t, int a_T, int a_K, \
+        int a_M, int a_tiles_k, int a_round_sf, int a_use_clamp, float a_clamp
+#define TK_PC_KERNEL_UNPACK \
+    const PerChannelParams p{a_x, a_x_sf, a_p2t, a_out, a_out_sf, a_T, a_K, a_M, a_tiles_k, a_round_sf, a_use_clamp, a_clamp}
+#define TK_PC_LAUNCH_ARGS(p) \
+    (p).x, (p).out, (p).out_sf, (p).x_sf, (p).pos_to_token, (p).num_tokens, (p).K, (p).M, (p).tiles_k, (p).round_sf, (p).use_clamp, (p).clamp
+
+template <int MODE> struct PcRaw { typedef Raw8<bf16_t> type; };
+template <> struct PcRaw<PC_E4M3> { typedef Raw8<e4m3in_t> type; };
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{a, b}), bf16x2));
+}
+
+template <int MODE, int NPT, bool TRANS, bool GATHER>
+__global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_KERNEL_ARGS) {
+    TK_PC_KERNEL_UNPACK;
+    constexpr int NB = kPcTileM / NPT;          // scale blocks per tile along the tokens: 1 or 4
+    typedef typename PcRaw<MODE>::type Raw;
+    __shared__ __attribute__((aligned(16))) float part[16][kPcTileK];    // [wave * 2 + half][column]
+    __shared__ __attribute__((aligned(16))) float inv_s[NB][kPcTileK];
+    __shared__ __attribute__((aligned(16))) uint8_t turned[TRANS ? kPcTileK * kPcPitch : 16];
+
+    const int tile_m = blockIdx.x / p.tiles_k, tile_k = blockIdx.x - tile_m * p.tiles_k;
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const int half = lane >> 5, hl = lane & 31;
+    const int col0 = tile_k * kPcTileK, col = col0 + hl * 8;
+    const bool col_ok = col < p.K;
+    const int tok0 = tile_m * kPcTileM + wave * 16 + half * 8;
+    const bool rows_ok = tok0 < p.M;            // M is a multiple of 16: all 8 tokens of a lane or none
+    const int64_t in_ld = MODE == PC_SWIGLU ? 2 * (int64_t)p.K : p.K;
+    const float cl = p.use_clamp ? p.clamp : __builtin_inff();   // no clamp = clamp at infinity: no branch in the hot loop
+
+    // ---- load (and, for SwiGLU, activate) 8 tokens x 8 columns.  Whether a lane has anything to load
+    // does not depend on the token (M is a multiple of 16), so the loads sit in straight-line code
+    // under one branch; a gathered row with a negative index is read from row 0 and zeroed by value.
+    Raw raw[kPcRows];
+#pragma unroll
+    for (int r = 0; r < kPcRows; ++r) raw[r].zero();
+    if (rows_ok && col_ok) {
+#pragma unroll
+        for (int r = 0; r < kPcRows; ++r) {
+            int src = tok0 + r;
+            bool valid = true;
+            if constexpr (GATHER) {
+                src = p.pos_to_token[tok0 + r];
+                valid = src >= 0 && src < p.num_tokens;
+                src = valid ? src : 0;
+            }
+            if constexpr (MODE == PC_SWIGLU) {
+                const uint16_t *xr = reinterpret_cast<const uint16_t *>(p.x) + (int64_t)src * in_ld + col;
+                Raw8<bf16_t> rg, ru;
+                rg.load(xr);
+                ru.load(xr + p.K);
+                float g[8], u[8], a[8];
+                rg.get(g);
+                ru.get(u);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    g[i] = __builtin_fminf(g[i], cl);
+                    u[i] = __builtin_fminf(__builtin_fmaxf(u[i], -cl), cl);
+                    a[i] = silu_mul<bf16_t>(g[i], u[i]);
+                }
+                // the activation is rounded to bf16 before it is quantised, as in the reference
+                raw[r].w = u32x4{pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]), pack_bf16x2(a[4], a[5]), pack_bf16x2(a[6], a[7])};
+                // four tokens (eight loads) at a time: all sixteen loads at once would not fit the registers
+                if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+            } else if constexpr (MODE == PC_E4M3) {
+                raw[r].load(reinterpret_cast<const uint8_t *>(p.x) + (int64_t)src * in_ld + col);
+                raw[r].s = p.x_sf[(int64_t)src * (p.K >> 7) + (col >> 7)];
+                if (GATHER && !valid) { raw[r].w = u32x2{0u, 0u}; raw[r].s = 0.0f; }
+            } else {
+                raw[r].load(reinterpret_cast<const uint16_t *>(p.x) + (int64_t)src * in_ld + col);
+                if (GATHER && !valid) raw[r].zero();
+            }
+        }
+    }
+
+    // ---- |x| maxima down this lane's 8 columns
+    float m[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) m[j] = 0.0f;
+#pragma unroll
+    for (int r = 0; r < kPcRows; ++r) {
+        float v[8];
+        raw[r].get(v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) m[j] = __builtin_fmaxf(m[j], __builtin_fabsf(v[j]));
+    }
+    // the tile is unpacked a second time after the scales are known; without this the compiler keeps
+    // all 64 unpacked values alive across the two barriers instead
+#pragma unroll
+    for (int r = 0; r < kPcRows; ++r) asm volatile("" : "+v"(raw[r].w));
+    {
+        u32x4 *dst = reinterpret_cast<u32x4 *>(&part[wave * 2 + half][hl * 8]);
+        dst[0] = u32x4{f2u(m[0]), f2u(m[1]), f2u(m[2]), f2u(m[3])};
+        dst[1] = u32x4{f2u(m[4]), f2u(m[5]), f2u(m[6]), f2u(m[7])};
+    }
+    __syncthreads();
+
+    // ---- thread c: scale(s) of column c
+    if (threadIdx.x < kPcTileK) {
+        const int c = threadIdx.x;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            float a = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16 / NB; ++i) a = __builtin_fmaxf(a, part[b * (16 / NB) + i][c]);
+            const Scale sc = make_scale<448>(a, Fmt<TK_E4M3>::floor_, p.round_sf != 0);
+            inv_s[b][c] = sc.inv;
+            const int tok = tile_m * kPcTileM + b * NPT;
+            if (tok < p.M && col0 + c < p.K) st_stream4(p.out_sf + (int64_t)(tok / NPT) * p.K + col0 + c, f2u(sc.sf));
+        }
+    }
+    __syncthreads();
+
+    float inv[8];
+    {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(&inv_s[NB == 1 ? 0 : (wave >> 1)][hl * 8]);
+        const u32x4 a = src[0], b = src[1];
+        inv[0] = u2f(a.x); inv[1] = u2f(a.y); inv[2] = u2f(a.z); inv[3] = u2f(a.w);
+        inv[4] = u2f(b.x); inv[5] = u2f(b.y); inv[6] = u2f(b.z); inv[7] = u2f(b.w);
+    }
+
+    if constexpr (!TRANS) {
+#pragma unroll
+        for (int r = 0; r < kPcRows; ++r) {
+            float v[8], q[8];
+            raw[r].get(v);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j] = v[j] * inv[j];
+            if (rows_ok && col_ok) st_stream8(p.out + (int64_t)(tok0 + r) * p.K + col, pack_e4m3x8<false>(q));
+        }
+    } else {
+        // codes of 8 consecutive tokens per column: token pairs fill the 16-bit halves of 2 dwords
+        uint32_t acc[8][2];
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+            float v0[8], v1[8], v2[8], v3[8];
+            raw[4 * d].get(v0);
+            raw[4 * d + 1].get(v1);
+            raw[4 * d + 2].get(v2);
+            raw[4 * d + 3].get(v3);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int lo = __builtin_amdgcn_cvt_pk_fp8_f32(v0[j] * inv[j], v1[j] * inv[j], 0, false);
+                acc[j][d] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(v2[j] * inv[j], v3[j] * inv[j], lo, true);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            *reinterpret_cast<u32x2 *>(&turned[(hl * 8 + j) * kPcPitch + wave * 16 + half * 8]) = u32x2{acc[j][0], acc[j][1]};
+        __syncthreads();
+        // 8 lanes x 16 bytes = the 128 tokens of one output row; a wave stores 8 rows per step
+        const int chunk = threadIdx.x & 7;
+        const int tok = tile_m * kPcTileM + chunk * 16;
+#pragma unroll
+        for (int i = 0; i < kPcTileK / 64; ++i) {
+            const int h = (threadIdx.x >> 3) + 64 * i;
+            if (col0 + h < p.K && tok < p.M) {
+                const u32x4 d = *reinterpret_cast<const u32x4 *>(&turned[h * kPcPitch + chunk * 16]);
+                __builtin_nontemporal_store(d, reinterpret_cast<u32x4 *>(p.out + (int64_t)(col0 + h) * p.M + tok));
+            }
+        }
+    }
+}
+
+template <int MODE, int NPT>
+static void launch_per_channel_2(const PerChannelParams &p, bool transpose, hipStream_t stream) {
+    const int tiles_m = (p.M + kPcTileM - 1) / kPcTileM;
+    const dim3 grid((unsigned)(tiles_m * p.tiles_k)), block(kPcThreads);
+#define TK_PC_LAUNCH(T, G) \
+    hipLaunchKernelGGL((per_channel_cast_kernel<MODE, NPT, T, G>), grid, block, 0, stream, TK_PC_LAUNCH_ARGS(p))
+    if constexpr (MODE == PC_SWIGLU) {
+        if (transpose) TK_PC_LAUNCH(true, false);
+        else TK_PC_LAUNCH(false, false);
+    } else if (p.pos_to_token) {
+        if (transpose) TK_PC_LAUNCH(true, true);
+        else TK_PC_LAUNCH(false, true);
+    } else {
+        if (transpose) TK_PC_LAUNCH(true, false);
+        else TK_PC_LAUNCH(false, false);
+    }
+#undef TK_PC_LAUNCH
+}
+
+template <int MODE>
+static hipError_t launch_per_channel(const PerChannelParams &p, int num_per_tokens, bool transpose, hipStream_t stream) {
+    if (num_per_tokens == 128) launch_per_channel_2<MODE, 128>(p, transpose, stream);
+    else launch_per_channel_2<MODE, 32>(p, transpose, stream);
+    return hipGetLastError();
+}
+
+}  // namespace tk
+
+using namespace tk;
+
+extern "C" int tk_check_per_channel_cast(const void *x, int x_dtype, const float *x_sf, int64_t num_tokens, int64_t K,
+                                         const int32_t *pos_to_token, int64_t M, const void *out, const float *out_sf,
+                                         int num_per_tokens, int round_sf, int transpose, int swiglu, int use_clamp,
+                                         float clamp) {
+    (void)round_sf;
+    (void)pos_to_token;
+    (void)transpose;
+    if (x_dtype != TK_BF16) return TK_ERR_BAD_DTYPE;
+    if (num_per_tokens != 32 && num_per_tokens != 128) return TK_ERR_BAD_GROUP;
+    if (num_tokens < 0 || M < 0 || K <= 0 || K % 8 != 0 || M % 16 != 0) return TK_ERR_BAD_SHAPE;
+    if (x_sf && (K % 128 != 0 || swiglu)) return TK_ERR_BAD_MODE;
+    if (!pos_to_token && num_tokens < M) return TK_ERR_BAD_SHAPE;
+    if (swiglu && pos_to_token) return TK_ERR_BAD_MODE;
+    if (use_clamp && (!swiglu || !(clamp == clamp))) return TK_ERR_BAD_VALUE;
+    if (num_tokens > INT32_MAX - 256 || M > INT32_MAX - 256 || K > (INT32_MAX - 1024) / 2) return TK_ERR_TOO_LARGE;
+    if (M == 0) return TK_OK;
+    if (!x || !out || !out_sf) return TK_ERR_NULL_POINTER;
+    if (!aligned_to(x, x_sf ? 8 : 16) || !aligned_to(out, transpose ? 16 : 8) || !aligned_to(out_sf, 4) || !aligned_to(x_sf, 4))
+        return TK_ERR_MISALIGNED;
+    const int64_t tiles = ((M + kPcTileM - 1) / kPcTileM) * ((K + kPcTileK - 1) / kPcTileK);
+    if (tiles > INT32_MAX - 8) return TK_ERR_TOO_LARGE;
+    return TK_OK;
+}
+
+extern "C" int tk_per_channel_cast(const void *x, int x_dtype, const float *x_sf, int64_t num_tokens, int64_t K,
+                                   const int32_t *pos_to_token, int64_t M, void *out, float *out_sf, int num_per_tokens,
+                                   int round_sf, int transpose, int swiglu, int use_clamp, float clamp, void *stream) {
+    const int rc = tk_check_per_channel_cast(x, x_dtype, x_sf, num_tokens, K, pos_to_token, M, out, out_sf, num_per_tokens,
+                                             round_sf, transpose, swiglu, use_clamp, clamp);
+    if (rc != TK_OK || M == 0) return rc;
+    PerChannelParams p;
+    p.x = x;
+    p.x_sf = x_sf;
+    p.pos_to_token = pos_to_token;
+    p.out = static_cast<uint8_t *>(out);
+    p.out_sf = out_sf;
+    p.num_tokens = (int)num_tokens;
+    p.K = (int)K;
+    p.M = (int)M;
+    p.tiles_k = (int)((K + kPcTileK - 1) / kPcTileK);
+    p.round_sf = round_sf;
+    p.use_clamp = use_clamp;
+    p.clamp = clamp;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (swiglu) e = launch_per_channel<PC_SWIGLU>(p, num_per_tokens, transpose != 0, s);
+    else if (x_sf) e = launch_per_channel<PC_E4M3>(p, num_per_tokens, transpose != 0, s);
+    else e = launch_per_channel<PC_BF16>(p, num_per_tokens, transpose != 0, s);
+    return (int)e;
+}

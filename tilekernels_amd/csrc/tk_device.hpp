@@ -124,6 +124,7 @@ template <> struct Raw8<e4m3in_t> {
         w = u32x2{0u, 0u};
         if (ok) load(p);
     }
+    __device__ __forceinline__ void zero() { w = u32x2{0u, 0u}; s = 0.0f; }
     __device__ __forceinline__ void get(float (&v)[8]) const {
         const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.x, false), b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.x, true);
         const f32x2 c = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.y, false), d = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.y, true);
