@@ -6,8 +6,8 @@
 Companion of bench.py (which measures the headline workload and keeps the driver's contract): the
 same method -- C-ABI calls on preallocated device buffers, buffer sets rotated past the 256 MB
 last-level cache, HIP events on the launch stream over the timed region -- applied to the
-dequantisation, the re-quantisation of quantised input, the MoE layout helpers and the fused SwiGLU
-backward.  `bytes` is the algorithmic HBM traffic of one call (inputs read once, outputs written
+dequantisation, the re-quantisation of quantised input, the MoE layout helpers, the fused SwiGLU
+backward and the per-channel cast family.  `bytes` is the algorithmic HBM traffic of one call (inputs read once, outputs written
 once); `frac` prices it against 8 TB/s.
 """
 import argparse
@@ -154,6 +154,34 @@ def op_swiglu_backward(group=128, rows=8192, hidden=2048):
     return build
 
 
+def op_per_channel(mode, transpose, num_per_tokens=128, rows=8192, hidden=4096):
+    """mode: 'bf16' (plain), 'e4m3' (FP8 input with 1x128 scales), 'swiglu' (bf16 [rows, 2*hidden] in front)."""
+    def build():
+        import tilekernels_amd as tk
+        from tilekernels_amd import _ffi
+        lib = _ffi.load()
+        M, K = rows, hidden
+        x_sf = None
+        if mode == 'swiglu':
+            x = torch.randn((M, 2 * K), device='cuda', dtype=torch.bfloat16)
+        else:
+            x = torch.randn((M, K), device='cuda', dtype=torch.bfloat16)
+            if mode == 'e4m3':
+                x, x_sf = tk.quant.per_token_cast(x, 'e4m3', num_per_channels=128)
+        out = torch.empty((K, M) if transpose else (M, K), device='cuda', dtype=torch.float8_e4m3fn)
+        out_sf = torch.empty((M // num_per_tokens, K), device='cuda', dtype=torch.float32)
+        stream = _ffi.current_stream(out.device)
+
+        def launch():
+            rc = lib.tk_per_channel_cast(x.data_ptr(), 0, 0 if x_sf is None else x_sf.data_ptr(), M, K, 0, M, out.data_ptr(),
+                                         out_sf.data_ptr(), num_per_tokens, 1, int(transpose), int(mode == 'swiglu'), 0, 0.0,
+                                         stream)
+            assert rc == 0, rc
+        ts = [x, out, out_sf] + ([x_sf] if x_sf is not None else [])
+        return launch, nbytes(*ts), nbytes(*ts)
+    return build
+
+
 OPS = [
     Op('cast_back', 'cast_back e4m3 1x128 -> bf16, [8192,4096]', op_cast_back),
     Op('per_token_cast_quantized', 'per_token_cast of (e4m3 1x128) input -> e2m1 1x32, [8192,4096]', op_requant),
@@ -163,6 +191,16 @@ OPS = [
        op_swiglu_backward(128)),
     Op('swiglu_backward_and_per_token_cast_g32', 'swiglu_backward_and_per_token_cast 1x32 round_sf, x e4m3 [8192,4096]',
        op_swiglu_backward(32)),
+    Op('per_channel_cast', 'per_channel_cast 128x1 round_sf, bf16 [8192,4096]', op_per_channel('bf16', False)),
+    Op('per_channel_cast_fused_fp8_input', 'per_channel_cast_fused 128x1 of (e4m3 1x128) input, [8192,4096]',
+       op_per_channel('e4m3', False)),
+    Op('per_channel_cast_and_transpose', 'per_channel_cast_and_transpose 128x1 round_sf, bf16 [8192,4096] -> [4096,8192]',
+       op_per_channel('bf16', True)),
+    Op('swiglu_forward_and_per_channel_cast_and_transpose',
+       'swiglu_forward_and_per_channel_cast_and_transpose 128x1 round_sf, bf16 [8192,4096] -> [2048,8192]',
+       op_per_channel('swiglu', True, hidden=2048)),
+    Op('swiglu_forward_and_per_channel_cast', 'same without transpose, bf16 [8192,4096] -> [8192,2048]',
+       op_per_channel('swiglu', False, hidden=2048)),
 ]
 
 

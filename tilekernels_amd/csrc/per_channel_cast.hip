@@ -62,9 +62,12 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
     TK_PC_KERNEL_UNPACK;
     constexpr int NB = kPcTileM / NPT;          // scale blocks per tile along the tokens: 1 or 4
     typedef typename PcRaw<MODE>::type Raw;
-    __shared__ __attribute__((aligned(16))) float part[16][kPcTileK];    // [wave * 2 + half][column]
+    // the partial maxima are dead once the scales exist (second barrier), so the turned tile reuses their space
+    constexpr int kPartBytes = 16 * kPcTileK * 4, kTurnedBytes = TRANS ? kPcTileK * kPcPitch : 0;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kPartBytes > kTurnedBytes ? kPartBytes : kTurnedBytes];
     __shared__ __attribute__((aligned(16))) float inv_s[NB][kPcTileK];
-    __shared__ __attribute__((aligned(16))) uint8_t turned[TRANS ? kPcTileK * kPcPitch : 16];
+    float (*part)[kPcTileK] = reinterpret_cast<float (*)[kPcTileK]>(lds);    // [wave * 2 + half][column]
+    uint8_t *turned = lds;
 
     const int tile_m = blockIdx.x / p.tiles_k, tile_k = blockIdx.x - tile_m * p.tiles_k;
     const int lane = threadIdx.x & 63, wave = wave_id();
@@ -83,23 +86,21 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
 #pragma unroll
     for (int r = 0; r < kPcRows; ++r) raw[r].zero();
     if (rows_ok && col_ok) {
+        if constexpr (MODE == PC_SWIGLU) {
+            // all sixteen loads of the lane go out before the first activation is evaluated
+            Raw8<bf16_t> rg[kPcRows], ru[kPcRows];
 #pragma unroll
-        for (int r = 0; r < kPcRows; ++r) {
-            int src = tok0 + r;
-            bool valid = true;
-            if constexpr (GATHER) {
-                src = p.pos_to_token[tok0 + r];
-                valid = src >= 0 && src < p.num_tokens;
-                src = valid ? src : 0;
+            for (int r = 0; r < kPcRows; ++r) {
+                const uint16_t *xr = reinterpret_cast<const uint16_t *>(p.x) + (int64_t)(tok0 + r) * in_ld + col;
+                rg[r].load(xr);
+                ru[r].load(xr + p.K);
             }
-            if constexpr (MODE == PC_SWIGLU) {
-                const uint16_t *xr = reinterpret_cast<const uint16_t *>(p.x) + (int64_t)src * in_ld + col;
-                Raw8<bf16_t> rg, ru;
-                rg.load(xr);
-                ru.load(xr + p.K);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < kPcRows; ++r) {
                 float g[8], u[8], a[8];
-                rg.get(g);
-                ru.get(u);
+                rg[r].get(g);
+                ru[r].get(u);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     g[i] = __builtin_fminf(g[i], cl);
@@ -108,15 +109,25 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
                 }
                 // the activation is rounded to bf16 before it is quantised, as in the reference
                 raw[r].w = u32x4{pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]), pack_bf16x2(a[4], a[5]), pack_bf16x2(a[6], a[7])};
-                // four tokens (eight loads) at a time: all sixteen loads at once would not fit the registers
-                if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);
-            } else if constexpr (MODE == PC_E4M3) {
-                raw[r].load(reinterpret_cast<const uint8_t *>(p.x) + (int64_t)src * in_ld + col);
-                raw[r].s = p.x_sf[(int64_t)src * (p.K >> 7) + (col >> 7)];
-                if (GATHER && !valid) { raw[r].w = u32x2{0u, 0u}; raw[r].s = 0.0f; }
-            } else {
-                raw[r].load(reinterpret_cast<const uint16_t *>(p.x) + (int64_t)src * in_ld + col);
-                if (GATHER && !valid) raw[r].zero();
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < kPcRows; ++r) {
+                int src = tok0 + r;
+                bool valid = true;
+                if constexpr (GATHER) {
+                    src = p.pos_to_token[tok0 + r];
+                    valid = src >= 0 && src < p.num_tokens;
+                    src = valid ? src : 0;
+                }
+                if constexpr (MODE == PC_E4M3) {
+                    raw[r].load(reinterpret_cast<const uint8_t *>(p.x) + (int64_t)src * in_ld + col);
+                    raw[r].s = p.x_sf[(int64_t)src * (p.K >> 7) + (col >> 7)];
+                    if (GATHER && !valid) raw[r].zero();
+                } else {
+                    raw[r].load(reinterpret_cast<const uint16_t *>(p.x) + (int64_t)src * in_ld + col);
+                    if (GATHER && !valid) raw[r].zero();
+                }
             }
         }
     }
