@@ -69,7 +69,18 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
     float (*part)[kPcTileK] = reinterpret_cast<float (*)[kPcTileK]>(lds);    // [wave * 2 + half][column]
     uint8_t *turned = lds;
 
-    const int tile_m = blockIdx.x / p.tiles_k, tile_k = blockIdx.x - tile_m * p.tiles_k;
+    int tile_m = blockIdx.x / p.tiles_k, tile_k = blockIdx.x - tile_m * p.tiles_k;
+    if constexpr (MODE == PC_E4M3) {
+        // Workgroups are dealt to the 8 XCDs (each with its own L2) round-robin.  The tiles of one token
+        // range share the 128-byte lines of the input scales, so they are given to one XCD: 8 token
+        // ranges advance side by side, one per XCD.  (Without this the scale lines are fetched 8 times.)
+        const int tiles_m = (p.M + kPcTileM - 1) / kPcTileM, striped = (tiles_m / 8) * 8 * p.tiles_k;
+        if ((int)blockIdx.x < striped) {
+            const int q = blockIdx.x >> 3;
+            tile_k = q % p.tiles_k;
+            tile_m = (q / p.tiles_k) * 8 + (blockIdx.x & 7);
+        }
+    }
     const int lane = threadIdx.x & 63, wave = wave_id();
     const int half = lane >> 5, hl = lane & 31;
     const int col0 = tile_k * kPcTileK, col = col0 + hl * 8;
