@@ -137,6 +137,78 @@ def test_swiglu_validation(lib):
     assert check_sw(lib, sf_ld=3) == STRIDE
 
 
+def check_bwd(lib, x=P, x_sf=P, R=64, H=2048, group=128, go=P, w=P, ptt=P, t2p=P, nw=512, out=P, q=P, q_sf=P, xg=P, wg=P,
+              rnd=0, use_clamp=0, clamp=0.0):
+    return lib.tk_check_swiglu_backward_per_token_cast(x, x_sf, R, H, group, go, w, ptt, t2p, nw, out, q, q_sf, xg, wg, rnd,
+                                                       use_clamp, clamp)
+
+
+def test_swiglu_backward_validation(lib):
+    assert check_bwd(lib) == OK
+    assert check_bwd(lib, group=32) == OK
+    assert check_bwd(lib, group=64) == GROUP
+    assert check_bwd(lib, H=2080, group=128) == SHAPE                   # H % group
+    assert check_bwd(lib, R=-1) == SHAPE
+    assert check_bwd(lib, use_clamp=1, clamp=float('nan')) == VALUE
+    assert check_bwd(lib, go=0) == NULLP
+    assert check_bwd(lib, wg=0) == NULLP                                # needed whenever there are (token, k) pairs
+    assert check_bwd(lib, R=0, x=0, x_sf=0, go=0, w=0, ptt=0, out=0, q=0, q_sf=0, xg=0) == OK   # no rows: only weight_grad
+    assert check_bwd(lib, R=0, nw=0, x=0, x_sf=0, go=0, w=0, ptt=0, t2p=0, out=0, q=0, q_sf=0, xg=0, wg=0) == OK
+    assert check_bwd(lib, go=P + 8) == ALIGN
+    assert check_bwd(lib, x=P + 4) == ALIGN
+    assert check_bwd(lib, R=2 ** 31) == LARGE
+
+
+def check_pc(lib, x=P, dt=0, x_sf=0, T=256, K=512, p2t=0, M=256, out=P, out_sf=P, npt=128, rnd=0, tr=0, sw=0, use_clamp=0,
+             clamp=0.0):
+    return lib.tk_check_per_channel_cast(x, dt, x_sf, T, K, p2t, M, out, out_sf, npt, rnd, tr, sw, use_clamp, clamp)
+
+
+def test_per_channel_cast_validation(lib):
+    assert check_pc(lib) == OK
+    assert check_pc(lib, npt=32, tr=1) == OK
+    assert check_pc(lib, npt=64) == GROUP
+    assert check_pc(lib, dt=1) == DTYPE                                 # bf16 (or FP8 + scales) only
+    assert check_pc(lib, M=250) == SHAPE                                # M % 16
+    assert check_pc(lib, K=20) == SHAPE                                 # K % 8
+    assert check_pc(lib, T=128) == SHAPE                                # without a gather the input must hold M rows
+    assert check_pc(lib, T=128, p2t=P) == OK
+    assert check_pc(lib, x_sf=P, K=192) == MODE                         # FP8 input comes with 1 x 128 scales
+    assert check_pc(lib, x_sf=P, K=256) == OK
+    assert check_pc(lib, x_sf=P, sw=1) == MODE
+    assert check_pc(lib, sw=1, p2t=P) == MODE
+    assert check_pc(lib, use_clamp=1, clamp=1.0) == VALUE               # the clamp belongs to the SwiGLU form
+    assert check_pc(lib, sw=1, use_clamp=1, clamp=1.0) == OK
+    assert check_pc(lib, x=P + 8) == ALIGN
+    assert check_pc(lib, x=P + 8, x_sf=P, K=256) == OK                  # codes need 8-byte alignment only
+    assert check_pc(lib, out=P + 8, tr=1) == ALIGN
+    assert check_pc(lib, out=0) == NULLP
+    assert check_pc(lib, M=0, T=0, x=0, out=0, out_sf=0) == OK
+
+
+def test_moe_layout_validation(lib):
+    ws = lib.tk_fused_mapping_workspace_bytes(4096, 8, 256)
+    assert ws > 0
+
+    def check_map(idx=P, T=4096, K=8, E=256, align=128, R=49152, ws_ptr=P, ws_bytes=ws, outs=P):
+        return lib.tk_check_get_fused_mapping(idx, T, K, E, align, R, outs, outs, outs, outs, outs, outs, outs, ws_ptr, ws_bytes)
+    assert check_map() == OK
+    assert check_map(E=2048) != OK                                      # more experts than the per-wave histogram holds
+    assert check_map(align=0) == VALUE
+    assert check_map(ws_bytes=ws - 4) == STRIDE                         # workspace too small
+    assert check_map(idx=0) == NULLP
+    assert check_map(outs=0) == NULLP
+
+    def check_exp(x=P, T=64, rb=4096, t2p=P, K=2, p2e=P, R=256, out=P, x_sf=0, cols=0, out_sf=0, ld=0, cm=0):
+        return lib.tk_check_expand_to_fused(x, T, rb, t2p, K, p2e, R, out, x_sf, cols, out_sf, ld, cm)
+    assert check_exp() == OK
+    assert check_exp(rb=4100) == ALIGN                                  # rows move as 16-byte pieces
+    assert check_exp(out=0) == NULLP
+    assert check_exp(x_sf=P, cols=32, out_sf=P, ld=32) == OK
+    assert check_exp(x_sf=P, cols=32, out_sf=P, ld=16) == STRIDE
+    assert check_exp(x_sf=P, cols=32, out_sf=0, ld=32) == NULLP
+
+
 def test_launching_entry_points_reject_before_touching_the_device(lib):
     """A rejected call returns the status from the same validation and launches nothing, so it is safe
     without a GPU."""
