@@ -38,7 +38,8 @@ class Op:
 
 
 def _sets_needed(footprint: int) -> int:
-    return max(3, -(-int(1.6 * LLC_BYTES) // max(footprint, 1)))
+    # small operators (the mapping) are latency-bound: a handful of sets is enough there
+    return min(16, max(3, -(-int(1.6 * LLC_BYTES) // max(footprint, 1))))
 
 
 def op_cast_back():

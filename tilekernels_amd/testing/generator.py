@@ -22,6 +22,43 @@ def generate_hidden_sizes(alignment: int = 64):
     return [h for h in (576, 2048, 2560, 3072, 4096, 6144, 7168) if h % alignment == 0]
 
 
+def generate_num_sms():
+    """Compute-unit limits to test with (tile_kernels/testing/generator.py:26-32)."""
+    from ..config import get_device_num_sms
+    n = get_device_num_sms()
+    base = [n - 20, n]
+    return [1] + base if _full_test() else base
+
+
+def generate_moe_params(is_benchmark: bool = False):
+    """Routing configurations of the reference's MoE-shaped tests, as seen by one expert-parallel rank
+    (tile_kernels/testing/generator.py:35-51): ``num_experts`` is the rank's local expert count."""
+    full = _full_test()
+    if full and not is_benchmark:
+        yield {'num_send_tokens': 0, 'num_topk': 1, 'num_experts': 1, 'num_ep_ranks': 1}
+    for num_tokens in (4001,):
+        for num_topk in (2, 6, 8, 9) + ((1, 7) if full else ()):
+            for num_experts in (72, 256) + ((288, 384) if full else ()):
+                for num_ep_ranks in (8, 64) + ((1, 72, 256) if full else ()):
+                    if num_experts % num_ep_ranks == 0:
+                        yield {'num_send_tokens': num_tokens, 'num_topk': num_topk,
+                               'num_experts': num_experts // num_ep_ranks, 'num_ep_ranks': num_ep_ranks}
+
+
+def generate_topk_idx(params: dict, device='cuda') -> torch.Tensor:
+    """Top-k expert ids of the tokens that reach this rank (tile_kernels/testing/generator.py:54-69):
+    every token of every rank picks ``num_topk`` of all experts; ids outside this rank's first
+    ``num_experts`` become -1 and tokens with no local expert are dropped.  int64 ``[tokens, num_topk]``."""
+    n, e, k, ranks = params['num_send_tokens'], params['num_experts'], params['num_topk'], params['num_ep_ranks']
+    if n == 0:
+        return torch.empty((0, k), dtype=torch.int64, device=device)
+    scores = torch.rand((n * ranks, e * ranks), dtype=torch.bfloat16, device=device)
+    topk_idx = torch.topk(scores, k=k, dim=-1, sorted=False).indices
+    away = topk_idx >= e
+    topk_idx = topk_idx.masked_fill(away, -1)
+    return topk_idx[~away.all(dim=1)].contiguous()
+
+
 def generate_moe_layout(num_tokens: int, num_experts: int, num_topk: int, alignment: int, generator: torch.Generator,
                         drop_fraction: float = 0.0):
     """Expert-major expanded layout of a top-k routed batch, built on the CPU.
