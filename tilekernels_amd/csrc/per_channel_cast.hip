@@ -25,7 +25,15 @@ namespace tk {
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kPcTileM = 128, kPcTileK = 256, kPcThreads = 512, kPcRows = 8;   // kPcRows tokens per lane
+// Tokens per lane.  Measured on MI355X at [8192, 4096] (us per call, 8 / 4 tokens per lane, i.e. 512 / 1024
+// threads per tile): plain 17.7 / 18.3, FP8 input 13.4 / 14.6, transposed 21.1 / 24.0, SwiGLU 17.3 / 18.0.
+#ifndef TK_PC_ROWS
+#define TK_PC_ROWS 8
+#endif
+constexpr int kPcTileM = 128, kPcTileK = 256;
+constexpr int kPcRows = TK_PC_ROWS;                      // consecutive tokens per lane (8 or 4)
+constexpr int kPcParts = kPcTileM / kPcRows;             // half-waves per tile = partial maxima per column
+constexpr int kPcThreads = 32 * kPcParts;                // 512 or 1024
 constexpr int kPcPitch = kPcTileM + 16;                                          // bytes per column in the turned tile
 
 enum { PC_BF16 = 0, PC_E4M3 = 1, PC_SWIGLU = 2 };
@@ -63,7 +71,7 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
     constexpr int NB = kPcTileM / NPT;          // scale blocks per tile along the tokens: 1 or 4
     typedef typename PcRaw<MODE>::type Raw;
     // the partial maxima are dead once the scales exist (second barrier), so the turned tile reuses their space
-    constexpr int kPartBytes = 16 * kPcTileK * 4, kTurnedBytes = TRANS ? kPcTileK * kPcPitch : 0;
+    constexpr int kPartBytes = kPcParts * kPcTileK * 4, kTurnedBytes = TRANS ? kPcTileK * kPcPitch : 0;
     __shared__ __attribute__((aligned(16))) uint8_t lds[kPartBytes > kTurnedBytes ? kPartBytes : kTurnedBytes];
     __shared__ __attribute__((aligned(16))) float inv_s[NB][kPcTileK];
     float (*part)[kPcTileK] = reinterpret_cast<float (*)[kPcTileK]>(lds);    // [wave * 2 + half][column]
@@ -85,7 +93,7 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
     const int half = lane >> 5, hl = lane & 31;
     const int col0 = tile_k * kPcTileK, col = col0 + hl * 8;
     const bool col_ok = col < p.K;
-    const int tok0 = tile_m * kPcTileM + wave * 16 + half * 8;
+    const int tok0 = tile_m * kPcTileM + (wave * 2 + half) * kPcRows;
     const bool rows_ok = tok0 < p.M;            // M is a multiple of 16: all 8 tokens of a lane or none
     const int64_t in_ld = MODE == PC_SWIGLU ? 2 * (int64_t)p.K : p.K;
     const float cl = p.use_clamp ? p.clamp : __builtin_inff();   // no clamp = clamp at infinity: no branch in the hot loop
@@ -172,7 +180,7 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
         for (int b = 0; b < NB; ++b) {
             float a = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 16 / NB; ++i) a = __builtin_fmaxf(a, part[b * (16 / NB) + i][c]);
+            for (int i = 0; i < kPcParts / NB; ++i) a = __builtin_fmaxf(a, part[b * (kPcParts / NB) + i][c]);
             const Scale sc = make_scale<448>(a, Fmt<TK_E4M3>::floor_, p.round_sf != 0);
             inv_s[b][c] = sc.inv;
             const int tok = tile_m * kPcTileM + b * NPT;
@@ -183,7 +191,7 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
 
     float inv[8];
     {
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(&inv_s[NB == 1 ? 0 : (wave >> 1)][hl * 8]);
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(&inv_s[NB == 1 ? 0 : (wave * 2 * kPcRows) / 32][hl * 8]);
         const u32x4 a = src[0], b = src[1];
         inv[0] = u2f(a.x); inv[1] = u2f(a.y); inv[2] = u2f(a.z); inv[3] = u2f(a.w);
         inv[4] = u2f(b.x); inv[5] = u2f(b.y); inv[6] = u2f(b.z); inv[7] = u2f(b.w);
@@ -199,10 +207,11 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
             if (rows_ok && col_ok) st_stream8(p.out + (int64_t)(tok0 + r) * p.K + col, pack_e4m3x8<false>(q));
         }
     } else {
-        // codes of 8 consecutive tokens per column: token pairs fill the 16-bit halves of 2 dwords
-        uint32_t acc[8][2];
+        // codes of the lane's consecutive tokens per column: token pairs fill the 16-bit halves of a dword
+        constexpr int ND = kPcRows / 4;
+        uint32_t acc[8][ND];
 #pragma unroll
-        for (int d = 0; d < 2; ++d) {
+        for (int d = 0; d < ND; ++d) {
             float v0[8], v1[8], v2[8], v3[8];
             raw[4 * d].get(v0);
             raw[4 * d + 1].get(v1);
@@ -215,15 +224,18 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
             }
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            *reinterpret_cast<u32x2 *>(&turned[(hl * 8 + j) * kPcPitch + wave * 16 + half * 8]) = u32x2{acc[j][0], acc[j][1]};
+        for (int j = 0; j < 8; ++j) {
+            uint8_t *dst = &turned[(hl * 8 + j) * kPcPitch + (wave * 2 + half) * kPcRows];
+            if constexpr (ND == 2) *reinterpret_cast<u32x2 *>(dst) = u32x2{acc[j][0], acc[j][ND - 1]};
+            else *reinterpret_cast<uint32_t *>(dst) = acc[j][0];
+        }
         __syncthreads();
         // 8 lanes x 16 bytes = the 128 tokens of one output row; a wave stores 8 rows per step
         const int chunk = threadIdx.x & 7;
         const int tok = tile_m * kPcTileM + chunk * 16;
 #pragma unroll
-        for (int i = 0; i < kPcTileK / 64; ++i) {
-            const int h = (threadIdx.x >> 3) + 64 * i;
+        for (int i = 0; i < kPcTileK / (kPcThreads / 8); ++i) {
+            const int h = (threadIdx.x >> 3) + (kPcThreads / 8) * i;
             if (col0 + h < p.K && tok < p.M) {
                 const u32x4 d = *reinterpret_cast<const u32x4 *>(&turned[h * kPcPitch + chunk * 16]);
                 __builtin_nontemporal_store(d, reinterpret_cast<u32x4 *>(p.out + (int64_t)(col0 + h) * p.M + tok));
