@@ -8,7 +8,7 @@ same method -- C-ABI calls on preallocated device buffers, buffer sets rotated p
 last-level cache, HIP events on the launch stream over the timed region -- applied to the
 dequantisation, the re-quantisation of quantised input, the MoE layout helpers, the fused SwiGLU
 backward and the per-channel cast family.  `bytes` is the algorithmic HBM traffic of one call (inputs read once, outputs written
-once); `frac` prices it against 8 TB/s.
+once); `frac` prices it against 8 TB/s; `cpu_baseline` times the CPU oracle on the same input.
 """
 import argparse
 import json
@@ -31,7 +31,7 @@ def nbytes(*tensors) -> int:
 
 class Op:
     """`build()` returns (callable launching one call on torch's current stream, algorithmic bytes,
-    footprint bytes of the buffer set)."""
+    footprint bytes of the buffer set, factory of a callable that runs the CPU oracle on the same input)."""
 
     def __init__(self, name, workload, build):
         self.name, self.workload, self.build = name, workload, build
@@ -55,7 +55,11 @@ def op_cast_back():
     def launch():
         rc = lib.tk_cast_back(codes.data_ptr(), 0, M, K, sf.data_ptr(), sf.stride(0), 0, 1, 128, out.data_ptr(), 0, stream)
         assert rc == 0, rc
-    return launch, nbytes(codes, sf, out), nbytes(codes, sf, out)
+    def cpu():
+        from oracle import torch_ref
+        xq = (codes.cpu(), sf.cpu())
+        return lambda: torch_ref.cast_back(xq, 'bf16', (1, 128))
+    return launch, nbytes(codes, sf, out), nbytes(codes, sf, out), cpu
 
 
 def op_requant():
@@ -74,7 +78,11 @@ def op_requant():
         rc = lib.tk_per_token_cast_quantized(codes.data_ptr(), 0, M, K, K, sf.data_ptr(), sf.stride(0), 0, 1, 128,
                                              out.data_ptr(), out_sf.data_ptr(), out_sf.stride(0), 1, 32, 0, 0, stream)
         assert rc == 0, rc
-    return launch, nbytes(codes, sf, out, out_sf), nbytes(codes, sf, out, out_sf)
+    def cpu():
+        from oracle import torch_ref
+        xq = (codes.cpu(), sf.cpu())
+        return lambda: torch_ref.cast(xq, 'e2m1', (1, 32), x_block_size=(1, 128))
+    return launch, nbytes(codes, sf, out, out_sf), nbytes(codes, sf, out, out_sf), cpu
 
 
 def _moe_maps(T=4096, K=8, E=256, alignment=128, seed=0):
@@ -102,7 +110,12 @@ def op_get_fused_mapping():
                                       ws.data_ptr(), ws_bytes, stream)
         assert rc == 0, rc
     b = nbytes(topk_idx, p2e, p2t, ptt, t2p, es, ee, npe)
-    return launch, b, b
+
+    def cpu():
+        from oracle import torch_ref
+        idx = topk_idx.cpu()
+        return lambda: torch_ref.get_fused_mapping(idx, E, alignment)
+    return launch, b, b, cpu
 
 
 def op_expand_to_fused():
@@ -120,7 +133,11 @@ def op_expand_to_fused():
         rc = lib.tk_expand_to_fused(x.data_ptr(), T, hidden * 2, t2p.data_ptr(), K, p2e.data_ptr(), R, out.data_ptr(),
                                     0, 0, 0, 0, 0, stream)
         assert rc == 0, rc
-    return launch, nbytes(x, out, t2p, p2e), nbytes(x, out, t2p, p2e)
+    def cpu():
+        from oracle import torch_ref
+        xc, tc, pc = x.cpu(), t2p.cpu(), p2e.cpu()
+        return lambda: torch_ref.expand_to_fused(xc, tc, pc)
+    return launch, nbytes(x, out, t2p, p2e), nbytes(x, out, t2p, p2e), cpu
 
 
 def op_swiglu_backward(group=128, rows=8192, hidden=2048):
@@ -151,7 +168,12 @@ def op_swiglu_backward(group=128, rows=8192, hidden=2048):
                                                        stream)
             assert rc == 0, rc
         b = nbytes(codes, sf, go, w, ptt, t2p, out, q, q_sf, xg, wg)
-        return launch, b, b
+
+        def cpu():
+            from oracle import torch_ref
+            xq, goc, wc, pc, tc = (codes.cpu(), sf.cpu()), go.cpu(), w.cpu(), ptt.cpu(), t2p.cpu().view(T, K)
+            return lambda: torch_ref.swiglu_backward_and_per_token_cast(xq, goc, wc, pc, tc, group, True, None)
+        return launch, b, b, cpu
     return build
 
 
@@ -179,7 +201,17 @@ def op_per_channel(mode, transpose, num_per_tokens=128, rows=8192, hidden=4096):
                                          stream)
             assert rc == 0, rc
         ts = [x, out, out_sf] + ([x_sf] if x_sf is not None else [])
-        return launch, nbytes(*ts), nbytes(*ts)
+
+        def cpu():
+            from oracle import torch_ref
+            xc = x.cpu()
+            if mode == 'swiglu':
+                return lambda: torch_ref.swiglu_forward_and_per_channel_cast_and_transpose(xc, num_per_tokens, True, not transpose)
+            xin = (xc, x_sf.cpu()) if mode == 'e4m3' else xc
+            if transpose:
+                return lambda: torch_ref.per_channel_cast_and_transpose(xin, num_per_tokens, True)
+            return lambda: torch_ref.per_channel_cast_fused(xin, num_per_tokens, 128 if mode == 'e4m3' else None, True, None)
+        return launch, nbytes(*ts), nbytes(*ts), cpu
     return build
 
 
@@ -205,9 +237,25 @@ OPS = [
 ]
 
 
-def run(op: Op, steps: int, warmup: int) -> dict:
+def time_cpu(make) -> dict:
+    """The CPU oracle (test infrastructure: a restatement of the reference's torch implementation) on the
+    host cores for the same workload: one warm-up call, then two timed calls, the faster one reported."""
+    import time
+    threads = min(16, os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    fn = make()
+    fn()
+    best = float('inf')
+    for _ in range(2):
+        t0 = time.perf_counter()
+        fn()
+        best = min(best, time.perf_counter() - t0)
+    return {'ms_per_call': round(best * 1e3, 2), 'cores': threads, 'kind': 'port'}
+
+
+def run(op: Op, steps: int, warmup: int, with_cpu: bool) -> dict:
     sets = []
-    launch, algo, footprint = op.build()
+    launch, algo, footprint, make_cpu = op.build()
     sets.append(launch)
     for _ in range(_sets_needed(footprint) - 1):
         sets.append(op.build()[0])
@@ -223,8 +271,11 @@ def run(op: Op, steps: int, warmup: int) -> dict:
     torch.cuda.synchronize()
     us = e0.elapsed_time(e1) * 1e3 / steps
     gbs = algo / us / 1e3
-    return {'op': op.name, 'workload': op.workload, 'us_per_call': round(us, 2), 'bytes': algo, 'GB/s': round(gbs, 1),
-            'frac': round(gbs / HBM_PEAK_GBS, 4), 'buffer_sets': n, 'steps': steps, 'warmup': warmup}
+    rec = {'op': op.name, 'workload': op.workload, 'us_per_call': round(us, 2), 'bytes': algo, 'GB/s': round(gbs, 1),
+           'frac': round(gbs / HBM_PEAK_GBS, 4), 'buffer_sets': n, 'steps': steps, 'warmup': warmup}
+    if with_cpu:
+        rec['cpu_baseline'] = time_cpu(make_cpu)
+    return rec
 
 
 def main():
@@ -232,6 +283,7 @@ def main():
     ap.add_argument('--steps', type=int, default=2000)
     ap.add_argument('--warmup', type=int, default=1000)
     ap.add_argument('--only', type=str, default=None)
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU-oracle timing of each operator')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run plain 256 MiB device copies (reference point for hardware-counter runs)')
     a = ap.parse_args()
@@ -241,7 +293,7 @@ def main():
     for op in OPS:
         if a.only and a.only != op.name:
             continue
-        print(json.dumps(run(op, a.steps, a.warmup)), flush=True)
+        print(json.dumps(run(op, a.steps, a.warmup, not a.no_cpu)), flush=True)
         torch.cuda.empty_cache()
     if a.copy_calibration:
         from bench import copy_calibration
