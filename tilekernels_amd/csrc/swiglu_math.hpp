@@ -23,12 +23,21 @@ namespace tk {
 #define TK_SWIGLU_NEWTON 1
 #endif
 
+// max(g, -88) on the bit pattern: negative floats order like their patterns as unsigned integers, and
+// every non-negative float has a smaller pattern than -88, so one integer min does it.  (A float max
+// would cost a second instruction: its operand is an unpacked bit pattern that the compiler has to
+// canonicalise first.)  NaNs with the sign bit set come out as -88, other NaNs pass through.
+__device__ __forceinline__ float floor_at_minus_88(float g) {
+    const uint32_t b = f2u(g);
+    return u2f(b < 0xC2B00000u ? b : 0xC2B00000u);
+}
+
 template <typename InT> __device__ __forceinline__ float exp_neg(float g);
 
 template <> __device__ __forceinline__ float exp_neg<bf16_t>(float g) {
     constexpr float nh = -1.44268798828125f;             // -log2(e) cut to 15 significant bits (0xBFB8AA00)
     constexpr float nl_ln2 = -4.8884952e-06f;            // (-log2(e) - nh) * ln 2
-    const float gc = __builtin_fmaxf(g, -88.0f);
+    const float gc = floor_at_minus_88(g);
     const float e0 = __builtin_amdgcn_exp2f(gc * nh);    // exact product
     return __builtin_fmaf(e0, gc * nl_ln2, e0);
 }
@@ -36,7 +45,7 @@ template <> __device__ __forceinline__ float exp_neg<bf16_t>(float g) {
 template <> __device__ __forceinline__ float exp_neg<float>(float g) {
     constexpr float nh = -1.4426950216293335f;           // float(-log2 e)
     constexpr float nl = -1.9259629911266175e-8f;        // -log2 e - nh
-    const float gc = __builtin_fmaxf(g, -88.0f);
+    const float gc = floor_at_minus_88(g);
     const float th = gc * nh;
     const float tl = __builtin_fmaf(gc, nl, __builtin_fmaf(gc, nh, -th));
     const float e0 = __builtin_amdgcn_exp2f(th);
