@@ -26,7 +26,8 @@ def _topk_idx(T, K, E, drop=0.1, seed=0):
 
 
 @pytest.mark.parametrize('alignment', [16, 64, 128])
-@pytest.mark.parametrize('T,K,E', [(4001, 8, 256), (4001, 6, 72), (4001, 2, 9), (513, 9, 32), (7, 1, 1), (1, 2, 384), (64, 8, 1024)])
+@pytest.mark.parametrize('T,K,E', [(4001, 8, 256), (4001, 6, 72), (4001, 2, 9), (513, 9, 32), (7, 1, 1), (1, 2, 384), (64, 8, 1024),
+                                   (20001, 8, 256), (33000, 4, 9), (16384, 8, 64), (4001, 8, 768)])
 def test_get_fused_mapping(T, K, E, alignment):
     tk = _tk()
     topk_idx = _topk_idx(T, K, E, seed=T + K)
