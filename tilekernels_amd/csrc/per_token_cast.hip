@@ -167,10 +167,13 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERN
 
 // Rows per wave.  Measured on MI355X (us per call): bf16 [4096, 7168] -> E4M3 1x128 row-major scales
 // 18.1 / 16.3 / 17.0 for 1 / 2 / 4 rows; bf16 [16384, 7168] -> E2M1 1x32 packed scales 55.2 / 43.4 / 45.4.
-constexpr int kPerTokenRowsPerWave = 2;
+// Quantised input: a lane's 8 codes are only 8 (or 4) bytes, so a wave takes more rows to amortise
+// its fixed work; E4M3 1x128 [8192, 4096] -> E2M1 1x32: 14.3 / 12.0 / 12.2 for 2 / 4 / 8 rows.
+template <typename InT> constexpr int rows_per_wave() { return Elem<InT>::quantised ? 4 : 2; }
 
-template <typename InT, int G, int FMT, int RPW, bool WIDE>
-static void launch_per_token_4(PerTokenParams &p, hipStream_t stream) {
+template <typename InT, int G, int FMT, bool WIDE>
+static void launch_per_token_tiled(PerTokenParams &p, hipStream_t stream) {
+    constexpr int RPW = rows_per_wave<InT>();
     const int strips = (p.K + kStripCols - 1) / kStripCols;
     const int waves = WIDE ? wide_tile_waves(strips) : kWaves;
     const int rows = WIDE ? RPW : kWaves * RPW;
@@ -184,66 +187,29 @@ static void launch_per_token_4(PerTokenParams &p, hipStream_t stream) {
         hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, false>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
 }
 
-template <typename InT, int G, int FMT, int RPW>
-static void launch_per_token_3(PerTokenParams &p, hipStream_t stream) {
-    // a caller-supplied scale tensor is only read, so either tile shape does
-    if (p.sf.layout == TK_SF_ROW_F32) launch_per_token_4<InT, G, FMT, RPW, true>(p, stream);
-    else launch_per_token_4<InT, G, FMT, RPW, false>(p, stream);
-}
-
 template <typename InT, int G, int FMT>
-static void launch_per_token_2(PerTokenParams &p, hipStream_t stream) {
-    launch_per_token_3<InT, G, FMT, kPerTokenRowsPerWave>(p, stream);
+static void launch_per_token_group(PerTokenParams &p, hipStream_t stream) {
+    // a caller-supplied scale tensor is only read, so either tile shape does
+    if (p.sf.layout == TK_SF_ROW_F32) launch_per_token_tiled<InT, G, FMT, true>(p, stream);
+    else launch_per_token_tiled<InT, G, FMT, false>(p, stream);
 }
 
+// plain (bf16 / fp32) and quantised (codes + block scales) inputs alike; one scale per row (group == K
+// and not one of the tiled sizes) exists for plain inputs only
 template <typename InT, int FMT>
 static hipError_t launch_per_token(PerTokenParams &p, int group, hipStream_t stream) {
-    if (group == p.K && group != 16 && group != 32 && group != 64 && group != 128) {
-        hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT>), dim3(p.M), dim3(kThreads), 0, stream, TK_PT_LAUNCH_ARGS(p));
-        return hipGetLastError();
+    if constexpr (!Elem<InT>::quantised) {
+        if (group == p.K && group != 16 && group != 32 && group != 64 && group != 128) {
+            hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT>), dim3(p.M), dim3(kThreads), 0, stream, TK_PT_LAUNCH_ARGS(p));
+            return hipGetLastError();
+        }
     }
     switch (group) {
-        case 16: launch_per_token_2<InT, 16, FMT>(p, stream); break;
-        case 32: launch_per_token_2<InT, 32, FMT>(p, stream); break;
-        case 64: launch_per_token_2<InT, 64, FMT>(p, stream); break;
-        default: launch_per_token_2<InT, 128, FMT>(p, stream); break;
+        case 16: launch_per_token_group<InT, 16, FMT>(p, stream); break;
+        case 32: launch_per_token_group<InT, 32, FMT>(p, stream); break;
+        case 64: launch_per_token_group<InT, 64, FMT>(p, stream); break;
+        default: launch_per_token_group<InT, 128, FMT>(p, stream); break;
     }
-    return hipGetLastError();
-}
-
-// Quantised input (codes + block scales).
-template <typename InT, int G, int FMT, int RPW, bool WIDE>
-static void launch_per_token_requant_2(PerTokenParams &p, hipStream_t stream) {
-    const int strips = (p.K + kStripCols - 1) / kStripCols;
-    const int waves = WIDE ? wide_tile_waves(strips) : kWaves;
-    const int rows = WIDE ? RPW : kWaves * RPW;
-    const int cols = WIDE ? waves * kStripCols : kStripCols;
-    p.tiles_k = (p.K + cols - 1) / cols;
-    const dim3 grid((unsigned)(((p.M + rows - 1) / rows) * p.tiles_k)), block(64 * waves);
-    if (p.M % rows == 0 && p.K % cols == 0)
-        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, true>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
-    else
-        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, false>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
-}
-
-// Rows per wave for quantised input: a lane's 8 codes are only 8 (or 4) bytes, so a wave takes more
-// rows to amortise its fixed work.  Measured on MI355X, E4M3 1x128 [8192, 4096] -> E2M1 1x32
-// (us per call): 14.3 / 12.0 / 12.2 for 2 / 4 / 8 rows.
-constexpr int kRequantRowsPerWave = 4;
-
-template <typename InT, int FMT>
-static hipError_t launch_per_token_requant(PerTokenParams &p, int group, hipStream_t stream) {
-    const bool wide = p.sf.layout == TK_SF_ROW_F32;
-#define TK_RQ(G)                                                                                 \
-    if (wide) launch_per_token_requant_2<InT, G, FMT, kRequantRowsPerWave, true>(p, stream);     \
-    else launch_per_token_requant_2<InT, G, FMT, kRequantRowsPerWave, false>(p, stream)
-    switch (group) {
-        case 16: TK_RQ(16); break;
-        case 32: TK_RQ(32); break;
-        case 64: TK_RQ(64); break;
-        default: TK_RQ(128); break;
-    }
-#undef TK_RQ
     return hipGetLastError();
 }
 
@@ -365,8 +331,8 @@ extern "C" int tk_per_token_cast_quantized(const void *x, int x_fmt, int64_t M, 
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e;
     if (x_fmt == TK_E4M3)
-        e = fmt == TK_E4M3 ? launch_per_token_requant<e4m3in_t, TK_E4M3>(p, group, s) : launch_per_token_requant<e4m3in_t, TK_E2M1>(p, group, s);
+        e = fmt == TK_E4M3 ? launch_per_token<e4m3in_t, TK_E4M3>(p, group, s) : launch_per_token<e4m3in_t, TK_E2M1>(p, group, s);
     else
-        e = fmt == TK_E4M3 ? launch_per_token_requant<e2m1in_t, TK_E4M3>(p, group, s) : launch_per_token_requant<e2m1in_t, TK_E2M1>(p, group, s);
+        e = fmt == TK_E4M3 ? launch_per_token<e2m1in_t, TK_E4M3>(p, group, s) : launch_per_token<e2m1in_t, TK_E2M1>(p, group, s);
     return (int)e;
 }
