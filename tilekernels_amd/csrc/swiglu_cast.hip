@@ -18,6 +18,10 @@
 #define TK_TRACE(point)
 #endif
 
+#ifndef TK_MASK_BRANCHLESS
+#define TK_MASK_BRANCHLESS 1
+#endif
+
 namespace tk {
 
 struct SwigluParams {
@@ -114,14 +118,28 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_c
         TK_TRACE(0);
         Raw8<InT> rg[RPW], ru[RPW];
         bool live[RPW];   // wave-uniform
+        // the mask entries of all rows are fetched before the first of them is looked at: one scalar
+        // round trip in front of the loads instead of one per row
+        int expert[RPW];
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) expert[r] = (MASK && (FULL || row0 + r < p.R)) ? uniform_load(p.pos_to_expert + row0 + r) : 0;
+        if constexpr (MASK && RPW == 4)   // all four values must exist here, so their loads are issued together above
+            asm volatile("" ::"s"(expert[0]), "s"(expert[1]), "s"(expert[2]), "s"(expert[3]));
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
-            live[r] = FULL || row0 + r < p.R;
-            if (MASK && live[r]) live[r] = uniform_load(p.pos_to_expert + row0 + r) >= 0;
+            live[r] = (FULL || row0 + r < p.R) && expert[r] >= 0;
             const InT *xr = x + (int64_t)r * (2 * (int64_t)p.H);
             if (FULL && !MASK) {
                 rg[r].load(xr);
                 ru[r].load(xr + p.H);
+            } else if (FULL && MASK && TK_MASK_BRANCHLESS) {
+                // no branch around the loads (a branch would make the compiler wait for all eight loads
+                // before the first row is evaluated): a padding row reads the first bytes of the matrix,
+                // which every wave shares, and is cleared by value
+                const InT *src = live[r] ? xr : reinterpret_cast<const InT *>(p.x);
+                rg[r].load(src);
+                ru[r].load(live[r] ? xr + p.H : src);
+                if (!live[r]) { rg[r].zero(); ru[r].zero(); }
             } else {
                 rg[r].load(xr, live[r] && col_ok);
                 ru[r].load(xr + p.H, live[r] && col_ok);
