@@ -140,3 +140,32 @@ def test_per_channel_no_rows():
     assert tuple(codes.shape) == (0, 256) and tuple(sf.shape) == (0, 256)
     codes, sf = tk.quant.per_channel_cast_and_transpose(x, 'e4m3', 32)
     assert tuple(codes.shape) == (256, 0) and tuple(sf.shape) == (0, 256)
+
+
+@pytest.mark.parametrize('transpose', [False, True])
+@pytest.mark.parametrize('quantised', [False, True])
+def test_c_abi_combinations_the_wrappers_do_not_use(quantised, transpose):
+    """tk_per_channel_cast takes every combination of its flags; the Python wrappers only use the ones the
+    reference offers.  Here: 32 tokens per scale together with a gather whose length is 16 mod 32 (the
+    last scale block is half full), with and without FP8 input and transposed output."""
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    T, K, M = 200, 384, 16 * 21
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn((T, K), generator=g).to(torch.bfloat16)
+    pos = torch.randint(-1, T, (M,), generator=g, dtype=torch.int32)
+    xin = torch_ref.cast(x, 'e4m3', (1, 128)) if quantised else x
+    want_codes, want_sf = torch_ref.per_channel_cast_fused(xin, 32, 128 if quantised else None, False, pos)
+    if transpose:
+        want_codes = want_codes.T.contiguous()
+    xd = xin[0].cuda() if quantised else xin.cuda()
+    sfd = xin[1].cuda() if quantised else None
+    posd = pos.cuda()
+    out = torch.empty(tuple(want_codes.shape), dtype=torch.float8_e4m3fn, device='cuda')
+    out_sf = torch.empty(tuple(want_sf.shape), dtype=torch.float32, device='cuda')
+    rc = lib.tk_per_channel_cast(xd.data_ptr(), 0, _ffi.ptr(sfd), T, K, posd.data_ptr(), M, out.data_ptr(), out_sf.data_ptr(),
+                                 32, 0, int(transpose), 0, 0, 0.0, _ffi.current_stream(out.device))
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    assert_same(out, want_codes, 'codes')
+    assert_same(out_sf, want_sf, 'scales')
