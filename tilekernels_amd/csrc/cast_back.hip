@@ -21,13 +21,16 @@ constexpr int kBackRowsPerWave = 2;
 // the line for 16 bytes of it); otherwise the 4 waves are stacked, 512 columns wide.
 template <typename InT, bool OUT_F32, bool WIDE, bool FULL>
 __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_back_kernel(const void *x, void *out, void *a_sf, int64_t a_sf_ld,
-                                                                                         int M, int K, int tiles_k, int a_sf_layout, int nm,
+                                                                                         int M, int K, int geom, int a_sf_layout, int nm,
                                                                                          int nk, int bm, int bk) {
     constexpr int RPW = kBackRowsPerWave, ROWS = WIDE ? RPW : kWaves * RPW;
     const SfRef sf{a_sf, a_sf_ld, a_sf_layout, nm, nk};
-    const int tile_m = blockIdx.x / tiles_k, tile_k = blockIdx.x - tile_m * tiles_k;
+    // geom: wide tiles: waves per tile, the tile index comes from a 2-D grid (x = row tile, y = column
+    // tile); otherwise the number of column tiles of a 1-D grid
+    const int tile_m = WIDE ? (int)blockIdx.x : (int)blockIdx.x / geom;
+    const int tile_k = WIDE ? (int)blockIdx.y : (int)blockIdx.x - tile_m * geom;
     const int lane = threadIdx.x & 63, wave = wave_id();
-    const int strip = WIDE ? tile_k * (int)(blockDim.x >> 6) + wave : tile_k;
+    const int strip = WIDE ? tile_k * geom + wave : tile_k;
     const int col = strip * kStripCols + lane * 8;
     const bool col_ok = FULL || col < K;
     const int row0 = tile_m * ROWS + (WIDE ? 0 : wave * RPW);
@@ -69,12 +72,14 @@ static void launch_cast_back_2(const void *x, void *out, const void *sf, int64_t
     const int cols = WIDE ? waves * kStripCols : kStripCols;
     const int tiles_m = (M + rows - 1) / rows, tiles_k = (K + cols - 1) / cols;
     const int nm = (M + bm - 1) / bm, nk = (K + bk - 1) / bk;
-    const dim3 grid((unsigned)(tiles_m * tiles_k)), block(64 * waves);
+    const dim3 block(64 * waves);
+    const dim3 grid = WIDE ? dim3((unsigned)tiles_m, (unsigned)tiles_k) : dim3((unsigned)(tiles_m * tiles_k));
+    const int geom = WIDE ? waves : tiles_k;
     void *sfp = const_cast<void *>(sf);
     if (M % rows == 0 && K % cols == 0)
-        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, true>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, tiles_k, sf_layout, nm, nk, bm, bk);
+        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, true>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, geom, sf_layout, nm, nk, bm, bk);
     else
-        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, false>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, tiles_k, sf_layout, nm, nk, bm, bk);
+        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, false>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, geom, sf_layout, nm, nk, bm, bk);
 }
 
 template <typename InT, bool OUT_F32>
@@ -105,6 +110,7 @@ extern "C" int tk_check_cast_back(const void *x, int x_fmt, int64_t M, int64_t K
     const int64_t need = x_sf_layout == TK_SF_ROW_F32 ? nk : (x_sf_layout == TK_SF_COL_F32 ? nm : 4 * nm);
     if (x_sf_ld < need) return TK_ERR_BAD_STRIDE;
     if (((M + 1) / 2) * ((K + kStripCols - 1) / kStripCols) > INT32_MAX - 8) return TK_ERR_TOO_LARGE;
+    if (K / (3 * kStripCols) > 65535) return TK_ERR_TOO_LARGE;   // column tiles of the wide layout ride on grid.y
     return TK_OK;
 }
 

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(THREADS) void per_block_cast_kernel(TK_PB_KERNEL_AR
     // partial maxima: one per (scale block, 16-row slot of the workgroup); no atomics, no zeroing
     __shared__ __attribute__((aligned(16))) uint32_t part[SUBM][SUBK][TR];
 
-    const int tile_m = blockIdx.x / p.tiles_k, tile_k = blockIdx.x - tile_m * p.tiles_k;
+    const int tile_m = blockIdx.y, tile_k = blockIdx.x;   // 2-D grid: no division on the way to the first load
 
     const int t = threadIdx.x >> 4, c = threadIdx.x & 15;
     const int col = tile_k * kBlockTile + c * 8;
@@ -125,7 +125,7 @@ constexpr int kPerBlockThreads = 512;
 
 template <typename InT, int FMT, int BM, int BK>
 static void launch_per_block_2(const PerBlockParams &p, hipStream_t stream) {
-    const dim3 grid((unsigned)(p.tiles_m * p.tiles_k)), block(kPerBlockThreads);
+    const dim3 grid((unsigned)p.tiles_k, (unsigned)p.tiles_m), block(kPerBlockThreads);
     if (p.M % kBlockTile == 0 && p.K % kBlockTile == 0)
         hipLaunchKernelGGL((per_block_cast_kernel<InT, FMT, BM, BK, kPerBlockThreads, true>), grid, block, 0, stream, TK_PB_LAUNCH_ARGS(p));
     else
@@ -164,7 +164,7 @@ extern "C" int tk_check_per_block_cast(const void *x, int x_dtype, int64_t M, in
     const int64_t need = sf_layout == TK_SF_ROW_F32 ? nk : (sf_layout == TK_SF_COL_F32 ? nm : 4 * nm);
     if (sf_ld < need) return TK_ERR_BAD_STRIDE;
     const int64_t tiles = ((M + kBlockTile - 1) / kBlockTile) * ((K + kBlockTile - 1) / kBlockTile);
-    if (tiles > INT32_MAX - 8) return TK_ERR_TOO_LARGE;
+    if (tiles > INT32_MAX - 8 || (M + kBlockTile - 1) / kBlockTile > 65535) return TK_ERR_TOO_LARGE;   // row tiles ride on grid.y
     return TK_OK;
 }
 

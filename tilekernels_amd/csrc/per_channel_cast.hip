@@ -77,8 +77,11 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
     float (*part)[kPcTileK] = reinterpret_cast<float (*)[kPcTileK]>(lds);    // [wave * 2 + half][column]
     uint8_t *turned = lds;
 
-    int tile_m = blockIdx.x / p.tiles_k, tile_k = blockIdx.x - tile_m * p.tiles_k;
+    // 2-D grid (x = column tile, y = token tile); the FP8-input mode runs on a 1-D grid that it reorders
+    int tile_m = blockIdx.y, tile_k = blockIdx.x;
     if constexpr (MODE == PC_E4M3) {
+        tile_m = blockIdx.x / p.tiles_k;
+        tile_k = blockIdx.x - tile_m * p.tiles_k;
         // Workgroups are dealt to the 8 XCDs (each with its own L2) round-robin.  The tiles of one token
         // range share the 128-byte lines of the input scales, so they are given to one XCD: 8 token
         // ranges advance side by side, one per XCD.  (Without this the scale lines are fetched 8 times.)
@@ -247,7 +250,8 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
 template <int MODE, int NPT>
 static void launch_per_channel_2(const PerChannelParams &p, bool transpose, hipStream_t stream) {
     const int tiles_m = (p.M + kPcTileM - 1) / kPcTileM;
-    const dim3 grid((unsigned)(tiles_m * p.tiles_k)), block(kPcThreads);
+    const dim3 block(kPcThreads);
+    const dim3 grid = MODE == PC_E4M3 ? dim3((unsigned)(tiles_m * p.tiles_k)) : dim3((unsigned)p.tiles_k, (unsigned)tiles_m);
 #define TK_PC_LAUNCH(T, G) \
     hipLaunchKernelGGL((per_channel_cast_kernel<MODE, NPT, T, G>), grid, block, 0, stream, TK_PC_LAUNCH_ARGS(p))
     if constexpr (MODE == PC_SWIGLU) {
@@ -294,7 +298,7 @@ extern "C" int tk_check_per_channel_cast(const void *x, int x_dtype, const float
     if (!aligned_to(x, x_sf ? 8 : 16) || !aligned_to(out, transpose ? 16 : 8) || !aligned_to(out_sf, 4) || !aligned_to(x_sf, 4))
         return TK_ERR_MISALIGNED;
     const int64_t tiles = ((M + kPcTileM - 1) / kPcTileM) * ((K + kPcTileK - 1) / kPcTileK);
-    if (tiles > INT32_MAX - 8) return TK_ERR_TOO_LARGE;
+    if (tiles > INT32_MAX - 8 || (M + kPcTileM - 1) / kPcTileM > 65535) return TK_ERR_TOO_LARGE;   // token tiles ride on grid.y
     return TK_OK;
 }
 

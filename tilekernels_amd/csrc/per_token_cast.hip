@@ -22,7 +22,7 @@ struct PerTokenParams {
     SfRef sf;
     int64_t x_ld;     // (logical) elements between rows of x
     int M, K;
-    int tiles_k;
+    int geom;         // wide tiles: waves per tile (2-D grid: x = row tile, y = column tile); else column tiles (1-D grid)
     int round_sf, mode;
     SfRef xsf;        // quantised input only: its block scales ...
     int in_bm, in_bk; // ... and their block shape
@@ -31,14 +31,14 @@ struct PerTokenParams {
 // Parameters travel as individual scalars (16 dwords in all) so that they are preloaded into SGPRs
 // at wave start (the library is built with -amdgpu-kernarg-preload-count=16).
 #define TK_PT_KERNEL_ARGS                                                                                 \
-    const void *a_x, uint8_t *a_out, void *a_sf, int64_t a_sf_ld, int64_t a_x_ld, int a_M, int a_K, int a_tiles_k, \
+    const void *a_x, uint8_t *a_out, void *a_sf, int64_t a_sf_ld, int64_t a_x_ld, int a_M, int a_K, int a_geom, \
         int a_round_sf, int a_mode, int a_sf_layout, int a_nk, void *a_xsf, int64_t a_xsf_ld, int a_xsf_layout,      \
         int a_xsf_nm, int a_xsf_nk, int a_in_bm, int a_in_bk
 #define TK_PT_KERNEL_UNPACK                                                                                          \
-    const PerTokenParams p{a_x, a_out, SfRef{a_sf, a_sf_ld, a_sf_layout, a_M, a_nk}, a_x_ld, a_M, a_K, a_tiles_k,   \
+    const PerTokenParams p{a_x, a_out, SfRef{a_sf, a_sf_ld, a_sf_layout, a_M, a_nk}, a_x_ld, a_M, a_K, a_geom,   \
                            a_round_sf, a_mode, SfRef{a_xsf, a_xsf_ld, a_xsf_layout, a_xsf_nm, a_xsf_nk}, a_in_bm, a_in_bk}
 #define TK_PT_LAUNCH_ARGS(p)                                                                                         \
-    (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).x_ld, (p).M, (p).K, (p).tiles_k, (p).round_sf, (p).mode, (p).sf.layout, \
+    (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).x_ld, (p).M, (p).K, (p).geom, (p).round_sf, (p).mode, (p).sf.layout, \
         (p).sf.nk, (p).xsf.base, (p).xsf.ld, (p).xsf.layout, (p).xsf.nm, (p).xsf.nk, (p).in_bm, (p).in_bk
 
 // Tile shapes (RPW = rows per wave):
@@ -54,11 +54,13 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
     constexpr int GPS = kStripCols / G;   // groups per 512-column strip
     constexpr int ROWS = WIDE ? RPW : kWaves * RPW;       // rows per tile
     constexpr int SGPR = WIDE ? kMaxWideWaves * GPS : GPS;   // staged groups per row (capacity)
-    const int nwaves = WIDE ? (int)(blockDim.x >> 6) : kWaves;
+    // everything on the way to the first load comes from the preloaded arguments and the workgroup ids
+    const int nwaves = WIDE ? p.geom : kWaves;
     using RS = RowScales<Fmt<FMT>::qmax, RPW, LPG>;
     __shared__ uint32_t stage[ROWS][SGPR];
 
-    const int tile_m = blockIdx.x / p.tiles_k, tile_k = blockIdx.x - tile_m * p.tiles_k;
+    const int tile_m = WIDE ? (int)blockIdx.x : (int)blockIdx.x / p.geom;
+    const int tile_k = WIDE ? (int)blockIdx.y : (int)blockIdx.x - tile_m * p.geom;
     const int lane = threadIdx.x & 63, wave = wave_id();
     const int strip = WIDE ? tile_k * nwaves + wave : tile_k;
     const int col = strip * kStripCols + lane * 8;
@@ -178,9 +180,10 @@ static void launch_per_token_tiled(PerTokenParams &p, hipStream_t stream) {
     const int waves = WIDE ? wide_tile_waves(strips) : kWaves;
     const int rows = WIDE ? RPW : kWaves * RPW;
     const int cols = WIDE ? waves * kStripCols : kStripCols;
-    const int tiles_m = (p.M + rows - 1) / rows;
-    p.tiles_k = (p.K + cols - 1) / cols;
-    const dim3 grid((unsigned)(tiles_m * p.tiles_k)), block(64 * waves);
+    const int tiles_m = (p.M + rows - 1) / rows, tiles_k = (p.K + cols - 1) / cols;
+    p.geom = WIDE ? waves : tiles_k;
+    const dim3 block(64 * waves);
+    const dim3 grid = WIDE ? dim3((unsigned)tiles_m, (unsigned)tiles_k) : dim3((unsigned)(tiles_m * tiles_k));
     if (p.M % rows == 0 && p.K % cols == 0)
         hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, true>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
     else
@@ -244,6 +247,7 @@ extern "C" int tk_check_per_token_cast(const void *x, int x_dtype, int64_t M, in
     const int64_t nk = (K + group - 1) / group;
     if (M * nk > INT32_MAX) return TK_ERR_TOO_LARGE;
     if (((M + 3) / 4) * ((K + kStripCols - 1) / kStripCols) > INT32_MAX) return TK_ERR_TOO_LARGE;   // tile count
+    if (K / (3 * kStripCols) > 65535) return TK_ERR_TOO_LARGE;                                      // column tiles ride on grid.y
     const int64_t need = sf_layout == TK_SF_ROW_F32 ? nk : (sf_layout == TK_SF_COL_F32 ? M : 4 * M);
     if (sf_ld < need) return TK_ERR_BAD_STRIDE;
     if (sf_layout == TK_SF_COL_UE8M0 && sf_ld % 4 != 0) return TK_ERR_MISALIGNED;
@@ -263,7 +267,7 @@ extern "C" int tk_per_token_cast(const void *x, int x_dtype, int64_t M, int64_t 
     p.x_ld = x_row_stride;
     p.M = (int)M;
     p.K = (int)K;
-    p.tiles_k = (int)((K + kStripCols - 1) / kStripCols);
+    p.geom = 0;
     p.round_sf = round_sf;
     p.mode = mode;
     p.xsf = SfRef{nullptr, 0, TK_SF_ROW_F32, 0, 0};
@@ -305,6 +309,7 @@ extern "C" int tk_check_per_token_cast_quantized(const void *x, int x_fmt, int64
     const int64_t xnm = (M + x_bm - 1) / x_bm, xnk = (K + x_bk - 1) / x_bk;
     const int64_t xneed = x_sf_layout == TK_SF_ROW_F32 ? xnk : (x_sf_layout == TK_SF_COL_F32 ? xnm : 4 * xnm);
     if (x_sf_ld < xneed) return TK_ERR_BAD_STRIDE;
+    if (K / (3 * kStripCols) > 65535) return TK_ERR_TOO_LARGE;   // column tiles ride on grid.y
     return TK_OK;
 }
 
@@ -322,7 +327,7 @@ extern "C" int tk_per_token_cast_quantized(const void *x, int x_fmt, int64_t M, 
     p.x_ld = x_row_stride;
     p.M = (int)M;
     p.K = (int)K;
-    p.tiles_k = 0;
+    p.geom = 0;
     p.round_sf = round_sf;
     p.mode = TK_CAST_AND_SF;
     p.xsf = SfRef{const_cast<void *>(x_sf), x_sf_ld, x_sf_layout, (int)((M + x_bm - 1) / x_bm), (int)((K + x_bk - 1) / x_bk)};

@@ -41,6 +41,15 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 constexpr int kBwdMaxWaves = 8;
 
+// Waves per workgroup for a row of `strips` 512-column strips: all of them up to 8; beyond that the
+// largest of 8..4 that divides the count (no idle wave in the last pass), else 8.
+__host__ __device__ inline int backward_waves(int strips) {
+    if (strips <= kBwdMaxWaves) return strips;
+    for (int w = kBwdMaxWaves; w >= 4; --w)
+        if (strips % w == 0) return w;
+    return kBwdMaxWaves;
+}
+
 // Kernel arguments, hottest first (the first 16 dwords are preloaded into SGPRs).
 #define TK_BWD_KERNEL_ARGS                                                                                      \
     const uint8_t *x, const float *x_sf, const uint16_t *grad_out, uint16_t *out, uint16_t *x_grad, uint8_t *q, \
@@ -56,20 +65,13 @@ __global__ __launch_bounds__(64 * kBwdMaxWaves) void swiglu_backward_kernel(TK_B
     __shared__ float part[kBwdMaxWaves][RPW];
 
     const int lane = threadIdx.x & 63, wave = wave_id();
-    const int nwaves = (int)(blockDim.x >> 6);
-
-    // weight_grad of the (token, k) pairs that have no row: grid-stride over the whole table
-    {
-        const int64_t step = (int64_t)gridDim.x * blockDim.x;
-        for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < num_weights; i += step)
-            if (t2p[i] < 0) weight_grad[i] = 0.0f;
-    }
+    const int strips = (H + kStripCols - 1) / kStripCols;
+    const int nwaves = backward_waves(strips);   // = blockDim.x / 64, without waiting for the dispatch packet
 
     const int row0 = blockIdx.x * RPW;
-    if (row0 >= R) return;
-    const int strips = (H + kStripCols - 1) / kStripCols;
     const int nsf = 2 * H / N, hsf = H / N;
 
+    if (row0 < R) {
     int index[RPW];      // wave-uniform
     float w[RPW], acc[RPW];
 #pragma unroll
@@ -174,15 +176,15 @@ __global__ __launch_bounds__(64 * kBwdMaxWaves) void swiglu_backward_kernel(TK_B
         const int idx = (FULL || row0 + r < R) ? ptt[row0 + r] : -1;
         if (idx >= 0 && idx < num_weights) weight_grad[idx] = s;
     }
-}
+    }   // row0 < R
 
-// Waves per workgroup for a row of `strips` 512-column strips: all of them up to 8; beyond that the
-// largest of 8..4 that divides the count (no idle wave in the last pass), else 8.
-static int backward_waves(int strips) {
-    if (strips <= kBwdMaxWaves) return strips;
-    for (int w = kBwdMaxWaves; w >= 4; --w)
-        if (strips % w == 0) return w;
-    return kBwdMaxWaves;
+    // weight_grad of the (token, k) pairs that have no row: grid-stride over the whole table.  Last, so
+    // that its arguments (beyond the preloaded ones) are not waited for in front of the row loads.
+    {
+        const int64_t step = (int64_t)gridDim.x * blockDim.x;
+        for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < num_weights; i += step)
+            if (t2p[i] < 0) weight_grad[i] = 0.0f;
+    }
 }
 
 constexpr int kBwdRowsPerGroup = 2;

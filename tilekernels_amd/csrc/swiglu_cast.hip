@@ -34,7 +34,7 @@ struct SwigluParams {
     unsigned long long *clamped_count;
     int64_t num_weights;
     int R, H;
-    int tiles_m, tiles_k;
+    int nwaves, tiles_k;   // waves of a wide tile; tiles along the columns
     int round_sf;
     float floor_;        // amax lower clamp
     float clamp;
@@ -44,14 +44,14 @@ struct SwigluParams {
 // kernel-argument segment are preloaded into SGPRs when a wave starts (the library is built with
 // -amdgpu-kernarg-preload-count=16), which takes a scalar-cache miss off the front of every wave.
 #define TK_SWIGLU_KERNEL_ARGS                                                                                      \
-    const void *a_x, uint8_t *a_out, void *a_sf, int64_t a_sf_ld, int a_R, int a_H, int a_tiles_m, int a_tiles_k, \
+    const void *a_x, uint8_t *a_out, void *a_sf, int64_t a_sf_ld, int a_R, int a_H, int a_nwaves, int a_tiles_k, \
         float a_floor, float a_clamp, int a_round_sf, int a_sf_layout, const int32_t *a_pe, const int32_t *a_ptt, \
         const float *a_w, unsigned long long *a_cnt, int64_t a_nw, int a_nk
 #define TK_SWIGLU_KERNEL_UNPACK                                                                            \
     const SwigluParams p{a_x, a_out, SfRef{a_sf, a_sf_ld, a_sf_layout, a_R, a_nk}, a_ptt, a_w, a_pe, a_cnt, \
-                         a_nw, a_R, a_H, a_tiles_m, a_tiles_k, a_round_sf, a_floor, a_clamp}
+                         a_nw, a_R, a_H, a_nwaves, a_tiles_k, a_round_sf, a_floor, a_clamp}
 #define TK_SWIGLU_LAUNCH_ARGS(p)                                                                                  \
-    (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).R, (p).H, (p).tiles_m, (p).tiles_k, (p).floor_, (p).clamp,       \
+    (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).R, (p).H, (p).nwaves, (p).tiles_k, (p).floor_, (p).clamp,       \
         (p).round_sf, (p).sf.layout, (p).pos_to_expert, (p).pos_to_token_topk, (p).topk_weights, (p).clamped_count, \
         (p).num_weights, (p).sf.nk
 
@@ -96,19 +96,24 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_c
     constexpr int GPS = kStripCols / 128;   // 4 groups per strip
     constexpr int ROWS = WIDE ? RPW : kWaves * RPW;
     constexpr int SGPR = WIDE ? kMaxWideWaves * GPS : GPS;   // staged groups per row (capacity)
-    const int nwaves = WIDE ? (int)(blockDim.x >> 6) : kWaves;
+    // The counting variant loops over tiles (its grid is capped so that few workgroups touch the global
+    // counters); every other variant has one workgroup per tile on a 2-D grid, which keeps integer
+    // divisions and further kernel-argument loads out of the path to the first memory load.
+    constexpr bool LOOP = CLAMP == 2;
+    const int nwaves = WIDE ? p.nwaves : kWaves;
     using RS = RowScales<448, RPW, 16>;
     __shared__ uint32_t stage[ROWS][SGPR];
 
-    const int total = p.tiles_m * p.tiles_k;
+    const int total = LOOP ? ((p.R + ROWS - 1) / ROWS) * p.tiles_k : 1;
     const int lane = threadIdx.x & 63, wave = wave_id();
     const bool has_weight = p.pos_to_token_topk != nullptr;
     const int own = lane & 15;
     const int srow = WIDE ? 0 : wave * RPW;
     ClampCounter<CLAMP> counter;
 
-    for (int tile = blockIdx.x; tile < total; tile += gridDim.x) {
-        const int tile_m = tile / p.tiles_k, tile_k = tile - tile_m * p.tiles_k;
+    for (int tile = LOOP ? (int)blockIdx.x : 0; tile < total; tile += LOOP ? (int)gridDim.x : 1) {
+        const int tile_m = LOOP ? tile / p.tiles_k : (int)blockIdx.x;
+        const int tile_k = LOOP ? tile - tile_m * p.tiles_k : (int)blockIdx.y;
         const int strip = WIDE ? tile_k * nwaves + wave : tile_k;
         const int col = strip * kStripCols + lane * 8;
         const bool col_ok = FULL || col < p.H;
@@ -199,7 +204,7 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_c
         __syncthreads();
         if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
         else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
-        if (gridDim.x < total) __syncthreads();   // stage is reused by the next tile
+        if (LOOP && (int)gridDim.x < total) __syncthreads();   // stage is reused by the next tile
     }
     counter.flush(p.clamped_count);
 }
@@ -272,10 +277,13 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
     const int waves = WIDE ? wide_tile_waves(strips) : kWaves;
     const int rows = WIDE ? RPW : kWaves * RPW;
     const int cols = WIDE ? waves * kStripCols : kStripCols;
-    p.tiles_m = (p.R + rows - 1) / rows;
+    const int tiles_m = (p.R + rows - 1) / rows;
     p.tiles_k = (p.H + cols - 1) / cols;
-    const int total = p.tiles_m * p.tiles_k;
-    const dim3 grid((unsigned)((max_blocks > 0 && max_blocks < total) ? max_blocks : total)), block(64 * waves);
+    p.nwaves = waves;
+    const int total = tiles_m * p.tiles_k;
+    const dim3 block(64 * waves);
+    const dim3 grid = CLAMP == 2 ? dim3((unsigned)((max_blocks > 0 && max_blocks < total) ? max_blocks : total))
+                                 : dim3((unsigned)tiles_m, (unsigned)p.tiles_k);
     const bool full = p.R % rows == 0 && p.H % cols == 0;
     if (p.pos_to_expert) {
         if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, true, true>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
@@ -338,7 +346,7 @@ extern "C" int tk_check_swiglu_per_token_cast(const void *x, int x_dtype, int64_
     if (sf_ld < need) return TK_ERR_BAD_STRIDE;
     if (sf_layout == TK_SF_COL_UE8M0 && sf_ld % 4 != 0) return TK_ERR_MISALIGNED;
     const int64_t tiles = ((R + 3) / 4) * ((H + kStripCols - 1) / kStripCols);
-    if (tiles > INT32_MAX - 8) return TK_ERR_TOO_LARGE;
+    if (tiles > INT32_MAX - 8 || H / kStripCols > 65535) return TK_ERR_TOO_LARGE;   // grid.y carries the column tiles
     return TK_OK;
 }
 
@@ -363,7 +371,7 @@ extern "C" int tk_swiglu_per_token_cast(const void *x, int x_dtype, int64_t R, i
     p.num_weights = num_weights;
     p.R = (int)R;
     p.H = (int)H;
-    p.tiles_m = p.tiles_k = 0;
+    p.nwaves = p.tiles_k = 0;
     p.round_sf = round_sf;
     p.floor_ = sf_clamp_min < 0.0f ? 1e-4f : sf_clamp_min;
     p.clamp = clamp;
