@@ -221,7 +221,7 @@ def cpu_baseline(w: Workload, budget_s: float = 12.0):
     return base, parity
 
 
-def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool):
+def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_streams: bool = True):
     w = Workload(cfg)
     wall, kern_us, per = time_gpu(w, steps, warmup)
     ms_per_step = wall / steps * 1e3
@@ -241,10 +241,11 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool):
                      'single_launch_us_median': round(statistics.median(per), 3), 'single_launch_us_min': round(min(per), 3)},
     }
     # informational: what the same entry point sustains when independent calls overlap
-    us2 = time_two_streams(w, steps)
-    line['two_streams'] = {'us_per_call': round(us2, 3), 'GBps': round(w.bytes / us2 / 1e3, 1),
-                           'pct_of_hbm_peak': round(w.bytes / us2 / 1e3 / HBM_PEAK_GBS * 100, 2),
-                           'note': 'calls alternate over two HIP streams; not used for value'}
+    if with_two_streams:
+        us2 = time_two_streams(w, steps)
+        line['two_streams'] = {'us_per_call': round(us2, 3), 'GBps': round(w.bytes / us2 / 1e3, 1),
+                               'pct_of_hbm_peak': round(w.bytes / us2 / 1e3 / HBM_PEAK_GBS * 100, 2),
+                               'note': 'calls alternate over two HIP streams; not used for value'}
     if with_cpu:
         line['cpu_baseline'], line['parity'] = cpu_baseline(w)
     return line
@@ -259,6 +260,9 @@ def main():
     ap.add_argument('--config', type=int, default=3, choices=sorted(WORKLOADS))
     ap.add_argument('--all-configs', action='store_true', help='also print one line per other configuration to stderr')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU-oracle baseline / parity leg')
+    ap.add_argument('--single-stream-only', action='store_true',
+                    help='skip the informational two-stream leg (for kernel traces: overlapping launches there would '
+                         'inflate the per-kernel durations)')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run plain device copies of known size (reference kernel for hardware-counter runs)')
     args = ap.parse_args()
@@ -270,8 +274,9 @@ def main():
     if args.all_configs:
         for cfg in sorted(WORKLOADS):
             if cfg != args.config:
-                print(json.dumps(bench_config(cfg, args.steps, args.warmup, not args.no_cpu)), file=sys.stderr, flush=True)
-    line = bench_config(args.config, args.steps, args.warmup, not args.no_cpu)
+                print(json.dumps(bench_config(cfg, args.steps, args.warmup, not args.no_cpu, not args.single_stream_only)),
+                      file=sys.stderr, flush=True)
+    line = bench_config(args.config, args.steps, args.warmup, not args.no_cpu, not args.single_stream_only)
     if args.copy_calibration:
         line.update(copy_calibration())
     print(json.dumps(line), flush=True)
