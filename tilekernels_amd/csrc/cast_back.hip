@@ -21,8 +21,8 @@ constexpr int kBackRowsPerWave = 2;
 // the line for 16 bytes of it); otherwise the 4 waves are stacked, 512 columns wide.
 template <typename InT, bool OUT_F32, bool WIDE, bool FULL>
 __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_back_kernel(const void *x, void *out, void *a_sf, int64_t a_sf_ld,
-                                                                                         int M, int K, int geom, int a_sf_layout, int nm,
-                                                                                         int nk, int bm, int bk) {
+                                                                                         int M, int K, int geom, int bm, int bk, int a_sf_layout,
+                                                                                         int nm, int nk) {
     constexpr int RPW = kBackRowsPerWave, ROWS = WIDE ? RPW : kWaves * RPW;
     const SfRef sf{a_sf, a_sf_ld, a_sf_layout, nm, nk};
     // geom: wide tiles: waves per tile, the tile index comes from a 2-D grid (x = row tile, y = column
@@ -77,9 +77,9 @@ static void launch_cast_back_2(const void *x, void *out, const void *sf, int64_t
     const int geom = WIDE ? waves : tiles_k;
     void *sfp = const_cast<void *>(sf);
     if (M % rows == 0 && K % cols == 0)
-        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, true>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, geom, sf_layout, nm, nk, bm, bk);
+        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, true>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, geom, bm, bk, sf_layout, nm, nk);
     else
-        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, false>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, geom, sf_layout, nm, nk, bm, bk);
+        hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, false>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, geom, bm, bk, sf_layout, nm, nk);
 }
 
 template <typename InT, bool OUT_F32>

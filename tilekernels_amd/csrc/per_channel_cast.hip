@@ -99,7 +99,6 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
     const int tok0 = tile_m * kPcTileM + (wave * 2 + half) * kPcRows;
     const bool rows_ok = tok0 < p.M;            // M is a multiple of 16: all 8 tokens of a lane or none
     const int64_t in_ld = MODE == PC_SWIGLU ? 2 * (int64_t)p.K : p.K;
-    const float cl = p.use_clamp ? p.clamp : __builtin_inff();   // no clamp = clamp at infinity: no branch in the hot loop
 
     // ---- load (and, for SwiGLU, activate) 8 tokens x 8 columns.  Whether a lane has anything to load
     // does not depend on the token (M is a multiple of 16), so the loads sit in straight-line code
@@ -118,6 +117,12 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
                 ru[r].load(xr + p.K);
             }
             __builtin_amdgcn_sched_barrier(0);
+            // the clamp arguments lie beyond the preloaded ones: touched only now, behind the loads.
+            // No clamp = clamp at infinity, so there is no branch in the hot loop.
+            float clamp_arg = p.clamp;
+            int use_clamp = p.use_clamp;
+            asm volatile("" : "+s"(clamp_arg), "+s"(use_clamp));
+            const float cl = use_clamp ? clamp_arg : __builtin_inff();
 #pragma unroll
             for (int r = 0; r < kPcRows; ++r) {
                 float g[8], u[8], a[8];

@@ -43,18 +43,20 @@ constexpr int kBwdMaxWaves = 8;
 
 // Waves per workgroup for a row of `strips` 512-column strips: all of them up to 8; beyond that the
 // largest of 8..4 that divides the count (no idle wave in the last pass), else 8.
-__host__ __device__ inline int backward_waves(int strips) {
+static int backward_waves(int strips) {
     if (strips <= kBwdMaxWaves) return strips;
     for (int w = kBwdMaxWaves; w >= 4; --w)
         if (strips % w == 0) return w;
     return kBwdMaxWaves;
 }
 
-// Kernel arguments, hottest first (the first 16 dwords are preloaded into SGPRs).
-#define TK_BWD_KERNEL_ARGS                                                                                      \
-    const uint8_t *x, const float *x_sf, const uint16_t *grad_out, uint16_t *out, uint16_t *x_grad, uint8_t *q, \
-        float *q_sf, int R, int H, float clamp, int round_sf, const int32_t *ptt, const float *weights,         \
-        float *weight_grad, const int32_t *t2p, int64_t num_weights
+// Kernel arguments, in the order they are needed: the first 14 dwords arrive preloaded in SGPRs and
+// hold everything the input addresses are made of; the rest is fetched from the argument buffer
+// while the first loads are in flight.
+#define TK_BWD_KERNEL_ARGS                                                                                       \
+    const uint8_t *x, const float *x_sf, const uint16_t *grad_out, int R, int H, int nwaves, int round_sf,        \
+        uint16_t *out, uint16_t *x_grad, uint8_t *q, float *q_sf, float clamp, const int32_t *ptt,               \
+        const float *weights, float *weight_grad, const int32_t *t2p, int64_t num_weights
 
 // N: columns per scale (32 or 128), of the input and of the quantised gradient alike.
 // CLAMP: the activation clamp is applied.  FULL: every wave's every strip is inside the matrix.
@@ -66,22 +68,14 @@ __global__ __launch_bounds__(64 * kBwdMaxWaves) void swiglu_backward_kernel(TK_B
 
     const int lane = threadIdx.x & 63, wave = wave_id();
     const int strips = (H + kStripCols - 1) / kStripCols;
-    const int nwaves = backward_waves(strips);   // = blockDim.x / 64, without waiting for the dispatch packet
 
     const int row0 = blockIdx.x * RPW;
     const int nsf = 2 * H / N, hsf = H / N;
 
     if (row0 < R) {
-    int index[RPW];      // wave-uniform
-    float w[RPW], acc[RPW];
+    float w[RPW], acc[RPW];   // w: wave-uniform
 #pragma unroll
-    for (int r = 0; r < RPW; ++r) {
-        const bool row_ok = FULL || row0 + r < R;
-        index[r] = row_ok ? uniform_load(ptt + row0 + r) : -1;
-        if (index[r] >= num_weights) index[r] = -1;
-        w[r] = index[r] >= 0 ? uniform_load(weights + index[r]) : 0.0f;
-        acc[r] = 0.0f;
-    }
+    for (int r = 0; r < RPW; ++r) w[r] = acc[r] = 0.0f;
 
     for (int strip = wave; strip < strips; strip += nwaves) {
         const int col = strip * kStripCols + lane * 8;
@@ -100,6 +94,22 @@ __global__ __launch_bounds__(64 * kBwdMaxWaves) void swiglu_backward_kernel(TK_B
             rgo[r].load(grad_out + row * (int64_t)H + col, ok);
             rg[r].s = ok ? x_sf[row * nsf + grp] : 0.0f;
             ru[r].s = ok ? x_sf[row * nsf + hsf + grp] : 0.0f;
+        }
+
+        // the rows' routing weights: two dependent scalar round trips, started only now that the
+        // strip's loads are in flight (the barrier keeps the compiler from hoisting them in front)
+        // arguments beyond the preloaded ones are first touched here, behind the loads: passing them
+        // through an empty asm keeps the address arithmetic built on them (which is loop-invariant) from
+        // being hoisted, together with the wait for their arrival, in front of the first strip's loads
+        asm volatile("" : "+s"(q), "+s"(q_sf), "+s"(clamp), "+s"(ptt), "+s"(weights));
+        if (strip == wave) {
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int r = 0; r < RPW; ++r) {
+                int idx = (FULL || row0 + r < R) ? uniform_load(ptt + row0 + r) : -1;
+                if (idx >= num_weights) idx = -1;
+                w[r] = idx >= 0 ? uniform_load(weights + idx) : 0.0f;
+            }
         }
 
         float dg[RPW][8], du[RPW][8], amax[2 * RPW];
@@ -216,7 +226,7 @@ static hipError_t launch_backward(const BackwardArgs &a, hipStream_t stream) {
     const dim3 grid((unsigned)blocks), block(64 * waves);
 #define TK_BWD_LAUNCH(F)                                                                                            \
     hipLaunchKernelGGL((swiglu_backward_kernel<N, CLAMP, RPW, F>), grid, block, 0, stream, a.x, a.x_sf, a.grad_out, \
-                       a.out, a.x_grad, a.q, a.q_sf, a.R, a.H, a.clamp, a.round_sf, a.ptt, a.weights, a.weight_grad, \
+                       a.R, a.H, waves, a.round_sf, a.out, a.x_grad, a.q, a.q_sf, a.clamp, a.ptt, a.weights, a.weight_grad, \
                        a.t2p, a.num_weights)
     if (full) TK_BWD_LAUNCH(true);
     else TK_BWD_LAUNCH(false);

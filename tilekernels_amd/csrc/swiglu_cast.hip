@@ -40,19 +40,20 @@ struct SwigluParams {
     float clamp;
 };
 
-// The kernels take their parameters as individual scalars, hottest first: the first 16 dwords of the
-// kernel-argument segment are preloaded into SGPRs when a wave starts (the library is built with
-// -amdgpu-kernarg-preload-count=16), which takes a scalar-cache miss off the front of every wave.
+// The kernels take their parameters as individual scalars in the order they are needed: the leading
+// 14 dwords of the kernel-argument segment arrive preloaded in SGPRs when a wave starts (the library is
+// built with -amdgpu-kernarg-preload-count=16) and hold everything the input addresses are made of; the
+// others are fetched from the argument buffer (host memory) while the first loads are in flight.
 #define TK_SWIGLU_KERNEL_ARGS                                                                                      \
-    const void *a_x, uint8_t *a_out, void *a_sf, int64_t a_sf_ld, int a_R, int a_H, int a_nwaves, int a_tiles_k, \
-        float a_floor, float a_clamp, int a_round_sf, int a_sf_layout, const int32_t *a_pe, const int32_t *a_ptt, \
+    const void *a_x, const int32_t *a_pe, int a_R, int a_H, int a_nwaves, int a_tiles_k, uint8_t *a_out, void *a_sf, \
+        int64_t a_sf_ld, float a_floor, float a_clamp, int a_round_sf, int a_sf_layout, const int32_t *a_ptt,          \
         const float *a_w, unsigned long long *a_cnt, int64_t a_nw, int a_nk
 #define TK_SWIGLU_KERNEL_UNPACK                                                                            \
     const SwigluParams p{a_x, a_out, SfRef{a_sf, a_sf_ld, a_sf_layout, a_R, a_nk}, a_ptt, a_w, a_pe, a_cnt, \
                          a_nw, a_R, a_H, a_nwaves, a_tiles_k, a_round_sf, a_floor, a_clamp}
 #define TK_SWIGLU_LAUNCH_ARGS(p)                                                                                  \
-    (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).R, (p).H, (p).nwaves, (p).tiles_k, (p).floor_, (p).clamp,       \
-        (p).round_sf, (p).sf.layout, (p).pos_to_expert, (p).pos_to_token_topk, (p).topk_weights, (p).clamped_count, \
+    (p).x, (p).pos_to_expert, (p).R, (p).H, (p).nwaves, (p).tiles_k, (p).out, (p).sf.base, (p).sf.ld, (p).floor_,  \
+        (p).clamp, (p).round_sf, (p).sf.layout, (p).pos_to_token_topk, (p).topk_weights, (p).clamped_count,         \
         (p).num_weights, (p).sf.nk
 
 // CLAMP: 0 none, 1 clamp, 2 clamp and count
