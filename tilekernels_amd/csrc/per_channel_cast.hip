@@ -25,16 +25,20 @@ namespace tk {
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
-// Tokens per lane.  Measured on MI355X at [8192, 4096] (us per call, 8 / 4 tokens per lane, i.e. 512 / 1024
-// threads per tile): plain 17.7 / 18.3, FP8 input 13.4 / 14.6, transposed 21.1 / 24.0, SwiGLU 17.3 / 18.0.
-#ifndef TK_PC_ROWS
-#define TK_PC_ROWS 8
-#endif
 constexpr int kPcTileM = 128, kPcTileK = 256;
-constexpr int kPcRows = TK_PC_ROWS;                      // consecutive tokens per lane (8 or 4)
-constexpr int kPcParts = kPcTileM / kPcRows;             // half-waves per tile = partial maxima per column
-constexpr int kPcThreads = 32 * kPcParts;                // 512 or 1024
-constexpr int kPcPitch = kPcTileM + 16;                                          // bytes per column in the turned tile
+// Consecutive tokens per lane.  With 4 (1024 threads per tile) every mode measured slower on MI355X at
+// [8192, 4096]: plain 17.7 -> 18.3 us, FP8 input 13.4 -> 14.6, transposed 21.1 -> 24.0, SwiGLU 17.3 -> 18.0.
+constexpr int kPcRows = 8;
+constexpr int kPcParts = kPcTileM / kPcRows;             // half-waves per tile = partial maxima per column: 16
+constexpr int kPcThreads = 32 * kPcParts;                // 512
+// Turned tile in LDS: one row of 128 token bytes per column, rows 144 bytes apart.  A lane writes the 8
+// tokens it holds of column 8 hl + j as one 8-byte word; left at its natural place (8 part) the 32
+// lanes of a half-wave would meet in two of the 32 8-byte bank pairs (rows 8 x 144 bytes apart).  So
+// the 16-byte unit of a row is rotated by (hl >> 1) & 7 and the two halves of the unit are exchanged
+// when hl >= 16: with the row pitch supplying hl & 1, the five bits of hl land in five different bits
+// of the bank-pair index and a half-wave's writes touch every bank pair once.  Units stay whole, so
+// the reader still takes 16 bytes at a time.
+constexpr int kPcPitch = kPcTileM + 16;
 
 enum { PC_BF16 = 0, PC_E4M3 = 1, PC_SWIGLU = 2 };
 
@@ -215,11 +219,10 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
             if (rows_ok && col_ok) st_stream8(p.out + (int64_t)(tok0 + r) * p.K + col, pack_e4m3x8<false>(q));
         }
     } else {
-        // codes of the lane's consecutive tokens per column: token pairs fill the 16-bit halves of a dword
-        constexpr int ND = kPcRows / 4;
-        uint32_t acc[8][ND];
+        // codes of the lane's 8 consecutive tokens per column: token pairs fill the 16-bit halves of a dword
+        uint32_t acc[8][2];
 #pragma unroll
-        for (int d = 0; d < ND; ++d) {
+        for (int d = 0; d < 2; ++d) {
             float v0[8], v1[8], v2[8], v3[8];
             raw[4 * d].get(v0);
             raw[4 * d + 1].get(v1);
@@ -231,11 +234,12 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
                 acc[j][d] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(v2[j] * inv[j], v3[j] * inv[j], lo, true);
             }
         }
+        {
+            const int part = wave * 2 + half;
+            const int unit = ((part >> 1) + (hl >> 1)) & 7, low = (part & 1) ^ (hl >> 4);
+            uint8_t *dst = &turned[hl * 8 * kPcPitch + unit * 16 + low * 8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            uint8_t *dst = &turned[(hl * 8 + j) * kPcPitch + (wave * 2 + half) * kPcRows];
-            if constexpr (ND == 2) *reinterpret_cast<u32x2 *>(dst) = u32x2{acc[j][0], acc[j][ND - 1]};
-            else *reinterpret_cast<uint32_t *>(dst) = acc[j][0];
+            for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x2 *>(dst + j * kPcPitch) = u32x2{acc[j][0], acc[j][1]};
         }
         __syncthreads();
         // 8 lanes x 16 bytes = the 128 tokens of one output row; a wave stores 8 rows per step
@@ -245,7 +249,9 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
         for (int i = 0; i < kPcTileK / (kPcThreads / 8); ++i) {
             const int h = (threadIdx.x >> 3) + (kPcThreads / 8) * i;
             if (col0 + h < p.K && tok < p.M) {
-                const u32x4 d = *reinterpret_cast<const u32x4 *>(&turned[h * kPcPitch + chunk * 16]);
+                const int unit = (chunk + (h >> 4)) & 7;
+                u32x4 d = *reinterpret_cast<const u32x4 *>(&turned[h * kPcPitch + unit * 16]);
+                if (i >= 2) d = u32x4{d.z, d.w, d.x, d.y};          // rows of the lanes hl >= 16: h >= 128
                 __builtin_nontemporal_store(d, reinterpret_cast<u32x4 *>(p.out + (int64_t)(col0 + h) * p.M + tok));
             }
         }
@@ -256,6 +262,8 @@ template <int MODE, int NPT>
 static void launch_per_channel_2(const PerChannelParams &p, bool transpose, hipStream_t stream) {
     const int tiles_m = (p.M + kPcTileM - 1) / kPcTileM;
     const dim3 block(kPcThreads);
+    // (token tiles on x, so that successive workgroups write neighbouring pieces of the same transposed rows,
+    // measured slower: 19.7 -> 21.1 us transposed, 17.4 -> 20.3 us with SwiGLU)
     const dim3 grid = MODE == PC_E4M3 ? dim3((unsigned)(tiles_m * p.tiles_k)) : dim3((unsigned)p.tiles_k, (unsigned)tiles_m);
 #define TK_PC_LAUNCH(T, G) \
     hipLaunchKernelGGL((per_channel_cast_kernel<MODE, NPT, T, G>), grid, block, 0, stream, TK_PC_LAUNCH_ARGS(p))
