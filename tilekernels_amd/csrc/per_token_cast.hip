@@ -30,16 +30,19 @@ struct PerTokenParams {
 
 // Parameters travel as individual scalars (16 dwords in all) so that they are preloaded into SGPRs
 // at wave start (the library is built with -amdgpu-kernarg-preload-count=16).
-#define TK_PT_KERNEL_ARGS                                                                                 \
-    const void *a_x, uint8_t *a_out, void *a_sf, int64_t a_sf_ld, int64_t a_x_ld, int a_M, int a_K, int a_geom, \
-        int a_round_sf, int a_mode, int a_sf_layout, int a_nk, void *a_xsf, int64_t a_xsf_ld, int a_xsf_layout,      \
-        int a_xsf_nm, int a_xsf_nk, int a_in_bm, int a_in_bk
+// Arguments in the order they are needed: the first 14 dwords arrive preloaded in SGPRs and hold all that
+// the input addresses (codes and, for a quantised input, its scales) are made of; the others are fetched
+// from the argument buffer while the loads are in flight.
+#define TK_PT_KERNEL_ARGS                                                                                          \
+    const void *a_x, int64_t a_x_ld, void *a_xsf, int64_t a_xsf_ld, int a_M, int a_K, int a_geom, int a_xsf_layout,  \
+        int a_in_bm, int a_in_bk, uint8_t *a_out, void *a_sf, int64_t a_sf_ld, int a_round_sf, int a_mode,           \
+        int a_sf_layout, int a_nk, int a_xsf_nm, int a_xsf_nk
 #define TK_PT_KERNEL_UNPACK                                                                                          \
     const PerTokenParams p{a_x, a_out, SfRef{a_sf, a_sf_ld, a_sf_layout, a_M, a_nk}, a_x_ld, a_M, a_K, a_geom,   \
                            a_round_sf, a_mode, SfRef{a_xsf, a_xsf_ld, a_xsf_layout, a_xsf_nm, a_xsf_nk}, a_in_bm, a_in_bk}
-#define TK_PT_LAUNCH_ARGS(p)                                                                                         \
-    (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).x_ld, (p).M, (p).K, (p).geom, (p).round_sf, (p).mode, (p).sf.layout, \
-        (p).sf.nk, (p).xsf.base, (p).xsf.ld, (p).xsf.layout, (p).xsf.nm, (p).xsf.nk, (p).in_bm, (p).in_bk
+#define TK_PT_LAUNCH_ARGS(p)                                                                                        \
+    (p).x, (p).x_ld, (p).xsf.base, (p).xsf.ld, (p).M, (p).K, (p).geom, (p).xsf.layout, (p).in_bm, (p).in_bk, (p).out, \
+        (p).sf.base, (p).sf.ld, (p).round_sf, (p).mode, (p).sf.layout, (p).sf.nk, (p).xsf.nm, (p).xsf.nk
 
 // Tile shapes (RPW = rows per wave):
 //   WIDE  (row-major scales):      RPW rows x (W*512) columns, W = blockDim.x/64 waves side by side on the same rows;
