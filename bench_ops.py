@@ -6,6 +6,7 @@
 Companion of bench.py (which measures the headline workload and keeps the driver's contract): the
 same method -- C-ABI calls on preallocated device buffers, buffer sets rotated past the 256 MB
 last-level cache, HIP events on the launch stream over the timed region -- applied to the
+scale-only and given-scale variants of the casts, the weighted MoE form of the headline operator, the
 dequantisation, the re-quantisation of quantised input, the MoE layout helpers, the fused SwiGLU
 backward and the per-channel cast family.  `bytes` is the algorithmic HBM traffic of one call (inputs read once, outputs written
 once); `frac` prices it against 8 TB/s; `cpu_baseline` times the CPU oracle on the same input.
@@ -215,7 +216,113 @@ def op_per_channel(mode, transpose, num_per_tokens=128, rows=8192, hidden=4096):
     return build
 
 
+def op_cast_variant(kind, mode):
+    """The scale-only and given-scale variants of the two casts at their benchmark shapes.
+    kind: 'token' (bf16 [4096,7168], 1x128) or 'block' (bf16 [7168,2048], 128x128); mode: 'sf_only' or 'given_sf'."""
+    def build():
+        import tilekernels_amd as tk
+        from tilekernels_amd import _ffi
+        lib = _ffi.load()
+        M, K = (4096, 7168) if kind == 'token' else (7168, 2048)
+        x = torch.randn((M, K), device='cuda', dtype=torch.bfloat16)
+        if kind == 'token':
+            sf = tk.quant.per_token_cast_with_sf_only(x, 'e4m3', 128)
+        else:
+            sf = tk.quant.per_block_cast_with_sf_only(x, 'e4m3', (128, 128))
+        out = torch.empty((M, K), device='cuda', dtype=torch.float8_e4m3fn)
+        stream = _ffi.current_stream(x.device)
+        code = _ffi.TK_SF_ONLY if mode == 'sf_only' else _ffi.TK_CAST_GIVEN_SF
+        op = 0 if mode == 'sf_only' else out.data_ptr()
+
+        def launch():
+            if kind == 'token':
+                rc = lib.tk_per_token_cast(x.data_ptr(), _ffi.TK_BF16, M, K, K, op, sf.data_ptr(), sf.stride(0), _ffi.TK_E4M3, 128,
+                                           _ffi.TK_SF_ROW_F32, 0, code, stream)
+            else:
+                rc = lib.tk_per_block_cast(x.data_ptr(), _ffi.TK_BF16, M, K, op, sf.data_ptr(), sf.stride(0), _ffi.TK_E4M3, 128, 128,
+                                           _ffi.TK_SF_ROW_F32, 0, code, stream)
+            assert rc == 0, rc
+        ts = [x, sf] + ([out] if mode == 'given_sf' else [])
+
+        def cpu():
+            from oracle import torch_ref
+            xc, sc = x.cpu(), sf.cpu()
+            blk = (1, 128) if kind == 'token' else (128, 128)
+            if mode == 'sf_only':
+                return lambda: torch_ref.cast(xc, 'e4m3', blk)[1]      # the oracle has no scale-only mode
+            return lambda: torch_ref.cast(xc, 'e4m3', blk, sf=sc)
+        return launch, nbytes(*ts), nbytes(x, sf, out), cpu
+    return build
+
+
+def op_expand_to_fused_with_sf():
+    import tilekernels_amd as tk
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    T, K, hidden = 4096, 8, 4096
+    _, maps = _moe_maps(T, K)
+    p2e, t2p = maps[0], maps[3]
+    R = p2e.numel()
+    x, x_sf = tk.quant.per_token_cast(torch.randn((T, hidden), device='cuda', dtype=torch.bfloat16), 'e4m3', 128)
+    out = torch.empty((R, hidden), device='cuda', dtype=torch.float8_e4m3fn)
+    out_sf = torch.empty((R, hidden // 128), device='cuda', dtype=torch.float32)
+    stream = _ffi.current_stream(x.device)
+
+    def launch():
+        rc = lib.tk_expand_to_fused(x.data_ptr(), T, hidden, t2p.data_ptr(), K, p2e.data_ptr(), R, out.data_ptr(),
+                                    x_sf.data_ptr(), hidden // 128, out_sf.data_ptr(), hidden // 128, 0, stream)
+        assert rc == 0, rc
+    ts = [x, x_sf, out, out_sf, t2p, p2e]
+
+    def cpu():
+        from oracle import torch_ref
+        xq, tc, pc = (x.cpu(), x_sf.cpu()), t2p.cpu(), p2e.cpu()
+        return lambda: torch_ref.expand_to_fused_with_sf(xq, 128, tc, pc)
+    return launch, nbytes(*ts), nbytes(*ts), cpu
+
+
+def op_swiglu_weighted():
+    """The headline operator on the MoE-expanded batch with routing weights (bench.py's config 4 has the mask only)."""
+    import tilekernels_amd as tk
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    T, K, H = 4096, 8, 2048
+    _, maps = _moe_maps(T, K)
+    p2e, ptt = maps[0], maps[2]
+    R = p2e.numel()
+    x = torch.randn((R, 2 * H), device='cuda', dtype=torch.bfloat16)
+    w = torch.rand((T, K), device='cuda')
+    out = torch.empty((R, H), device='cuda', dtype=torch.float8_e4m3fn)
+    sf = torch.empty((R, H // 128), device='cuda', dtype=torch.float32)
+    stream = _ffi.current_stream(x.device)
+
+    def launch():
+        rc = lib.tk_swiglu_per_token_cast(x.data_ptr(), _ffi.TK_BF16, R, H, out.data_ptr(), sf.data_ptr(), H // 128, 128,
+                                          _ffi.TK_SF_ROW_F32, 0, -1.0, ptt.data_ptr(), w.data_ptr(), T * K, p2e.data_ptr(),
+                                          0, 0.0, 0, 0, stream)
+        assert rc == 0, rc
+    live = int((p2e >= 0).sum())
+    # padding rows are not read; their codes and scales are written
+    algo = live * 2 * H * 2 + nbytes(out, sf, p2e, ptt, w)
+
+    def cpu():
+        from oracle import torch_ref
+        xc, pc, tc, wc = x.cpu(), p2e.cpu(), ptt.cpu(), w.cpu()
+        return lambda: torch_ref.swiglu_forward_and_per_token_cast(xc, 'e4m3', 128, pos_to_token_topk=tc, topk_weights=wc, pos_to_expert=pc)
+    return launch, algo, nbytes(x, out, sf), cpu
+
+
 OPS = [
+    Op('per_token_cast_with_sf_only', 'per_token_cast_with_sf_only e4m3 1x128, bf16 [4096,7168]', op_cast_variant('token', 'sf_only')),
+    Op('per_token_cast_with_precomputed_sf', 'per_token_cast_with_precomputed_sf e4m3 1x128, bf16 [4096,7168]',
+       op_cast_variant('token', 'given_sf')),
+    Op('per_block_cast_with_sf_only', 'per_block_cast_with_sf_only e4m3 128x128, bf16 [7168,2048]', op_cast_variant('block', 'sf_only')),
+    Op('per_block_cast_with_precomputed_sf', 'per_block_cast_with_precomputed_sf e4m3 128x128, bf16 [7168,2048]',
+       op_cast_variant('block', 'given_sf')),
+    Op('swiglu_forward_and_per_token_cast_weighted',
+       'swiglu_forward_and_per_token_cast e4m3 1x128, MoE-expanded bf16 [R,4096] with mask and routing weights', op_swiglu_weighted),
+    Op('expand_to_fused_with_sf', 'expand_to_fused_with_sf e4m3 [4096,4096] + 1x128 scales -> [R,4096], top-8 of 256 experts, pad 128',
+       op_expand_to_fused_with_sf),
     Op('cast_back', 'cast_back e4m3 1x128 -> bf16, [8192,4096]', op_cast_back),
     Op('per_token_cast_quantized', 'per_token_cast of (e4m3 1x128) input -> e2m1 1x32, [8192,4096]', op_requant),
     Op('get_fused_mapping', 'get_fused_mapping 4096 tokens, top-8 of 256 experts, pad 128', op_get_fused_mapping),

@@ -22,7 +22,8 @@
  *   TK_SF_ROW_F32    fp32, element (m, k) at sf[m * sf_ld + k]
  *   TK_SF_COL_F32    fp32, element (m, k) at sf[k * sf_ld + m]         (sf_ld >= nm)
  *   TK_SF_COL_UE8M0  one biased-exponent byte per block, at
- *                    ((uint8_t*)sf)[(k / 4) * sf_ld + 4 * m + (k % 4)]  (sf_ld in BYTES, >= 4 * nm);
+ *                    ((uint8_t*)sf)[(k / 4) * sf_ld + 4 * m + (k % 4)]  (sf_ld in BYTES, >= 4 * nm, a
+ *                    multiple of 4: the storage is an array of 4-byte words, 4-byte aligned);
  *                    needs round_sf = 1.  In cast modes the bytes of a partly filled last word
  *                    (k >= nk) are written as 0.
  * (reference: get_sf_shape / store_sf / load_sf, tile_kernels/quant/common.py:130-138, 219-244).

@@ -105,7 +105,7 @@ extern "C" int tk_check_cast_back(const void *x, int x_fmt, int64_t M, int64_t K
     if (M == 0) return TK_OK;
     if (!x || !x_sf || !out) return TK_ERR_NULL_POINTER;
     if (!aligned_to(x, x_fmt == TK_E4M3 ? 8 : 4) || !aligned_to(out, 16)) return TK_ERR_MISALIGNED;
-    if (x_sf_layout != TK_SF_COL_UE8M0 && !aligned_to(x_sf, 4)) return TK_ERR_MISALIGNED;
+    if (!aligned_to(x_sf, 4) || (x_sf_layout == TK_SF_COL_UE8M0 && x_sf_ld % 4 != 0)) return TK_ERR_MISALIGNED;
     const int64_t nm = (M + bm - 1) / bm, nk = (K + bk - 1) / bk;
     const int64_t need = x_sf_layout == TK_SF_ROW_F32 ? nk : (x_sf_layout == TK_SF_COL_F32 ? nm : 4 * nm);
     if (x_sf_ld < need) return TK_ERR_BAD_STRIDE;

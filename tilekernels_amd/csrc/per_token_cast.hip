@@ -92,7 +92,7 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
             const bool ok = col_ok && (FULL || row0 + r < p.M);
-            inv[r] = 1.0f / (ok ? sf_load(p.sf, row0 + r, kgrp) : 1.0f);
+            inv[r] = 1.0f / (ok ? sf_load_select(p.sf, row0 + r, kgrp) : 1.0f);
         }
     } else {
         float amax[RPW];
@@ -303,7 +303,7 @@ extern "C" int tk_check_per_token_cast_quantized(const void *x, int x_fmt, int64
     const uintptr_t unit = x_fmt == TK_E4M3 ? 8 : 4;     // bytes a lane loads
     if (!aligned_to(x, unit) || x_row_stride % 8 != 0) return TK_ERR_MISALIGNED;
     if (!aligned_to(out, 8) || !aligned_to(sf, 4)) return TK_ERR_MISALIGNED;
-    if (x_sf_layout != TK_SF_COL_UE8M0 && !aligned_to(x_sf, 4)) return TK_ERR_MISALIGNED;
+    if (!aligned_to(x_sf, 4) || (x_sf_layout == TK_SF_COL_UE8M0 && x_sf_ld % 4 != 0)) return TK_ERR_MISALIGNED;
     const int64_t nk = (K + group - 1) / group;
     if (M * nk > INT32_MAX) return TK_ERR_TOO_LARGE;
     const int64_t need = sf_layout == TK_SF_ROW_F32 ? nk : (sf_layout == TK_SF_COL_F32 ? M : 4 * M);

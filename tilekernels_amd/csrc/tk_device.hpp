@@ -325,6 +325,20 @@ __device__ __forceinline__ float sf_load(const SfRef &s, int m, int k) {
     return u2f(e << 23);
 }
 
+// The same without a branch: the layout only selects how the byte offset is formed, and the packed layout
+// is read as the aligned word that holds the byte (its storage consists of whole 4-byte words).  Loads of
+// several rows then go out back to back instead of one per branch.  Measured on MI355X: the given-scale
+// cast of bf16 [4096, 7168] 16.7 -> 16.0 us; the loaders of quantised input are better off with the
+// branches (re-quantisation of E4M3 [8192, 4096] 11.9 us against 12.3 us, dequantisation unchanged).
+__device__ __forceinline__ float sf_load_select(const SfRef &s, int m, int k) {
+    const bool packed = s.layout == TK_SF_COL_UE8M0;
+    const int64_t major = s.layout == TK_SF_ROW_F32 ? m : (packed ? k >> 2 : k);
+    const int64_t minor = s.layout == TK_SF_ROW_F32 ? k : m;
+    const int64_t off = packed ? major * s.ld + 4 * minor + (k & 3) : 4 * (major * s.ld + minor);
+    const uint32_t w = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint8_t *>(s.base) + (off & ~(int64_t)3));
+    return u2f(packed ? ((w >> (8 * (k & 3))) & 0xFFu) << 23 : w);
+}
+
 // store from a single lane; for the packed layout the lane that owns the last block of a row also
 // zeroes the unused bytes of that row's last word
 __device__ __forceinline__ void sf_store(const SfRef &s, int m, int k, const Scale &sc) {
