@@ -188,7 +188,8 @@ __global__ __launch_bounds__(kThreads) void fused_mapping_assign_kernel(const in
 // numbered 8 apart, which puts all of them on one XCD back to back.  (Measured for [4096, 4096] bf16,
 // top-8, random positions, 268 MB written: 50.6 us this way, 57 us with the copies of a chunk on
 // different XCDs, 61 us with one load and 8 stores per thread.)
-// The workgroups after those each look at one expanded row and zero it if it is padding.
+// The workgroups after those each look at a few consecutive expanded rows (8 KB worth) and zero the ones
+// that are padding.
 constexpr int kExpandChunk = kThreads * 16;
 
 // Non-temporal 16-byte stores: writing the same 268 MB as whole 8 KB rows per wave takes 52 us with them and
@@ -199,7 +200,7 @@ __global__ __launch_bounds__(kThreads) void expand_to_fused_kernel(const uint8_t
                                                                    int num_topk, int chunks, int copy_blocks, int num_tokens,
                                                                    int num_expanded, uint8_t *out, const int32_t *pos_to_expert,
                                                                    const uint32_t *x_sf, int sf_cols, uint32_t *out_sf,
-                                                                   int64_t out_sf_ld, int sf_col_major) {
+                                                                   int64_t out_sf_ld, int sf_col_major, int pad_rows) {
     const int b = blockIdx.x;
     if (b < copy_blocks) {
         // b = 8 * ((token group * chunks + chunk) * num_topk + k) + token within its group of 8
@@ -217,12 +218,14 @@ __global__ __launch_bounds__(kThreads) void expand_to_fused_kernel(const uint8_t
             for (int j = threadIdx.x; j < sf_cols; j += kThreads)
                 out_sf[sf_col_major ? (int64_t)j * out_sf_ld + p : (int64_t)p * out_sf_ld + j] = x_sf[(int64_t)t * sf_cols + j];
     } else {
-        const int r = b - copy_blocks;
-        if (uniform_load(pos_to_expert + r) >= 0) return;
-        uint8_t *dst = out + (int64_t)r * row_bytes;
-        for (int64_t off = (int64_t)threadIdx.x * 16; off < row_bytes; off += kExpandChunk) expand_store16(dst + off, u32x4{0u, 0u, 0u, 0u});
-        if (x_sf)
-            for (int j = threadIdx.x; j < sf_cols; j += kThreads) out_sf[sf_col_major ? (int64_t)j * out_sf_ld + r : (int64_t)r * out_sf_ld + j] = 0u;
+        const int r0 = (b - copy_blocks) * pad_rows;
+        for (int r = r0; r < r0 + pad_rows && r < num_expanded; ++r) {
+            if (uniform_load(pos_to_expert + r) >= 0) continue;
+            uint8_t *dst = out + (int64_t)r * row_bytes;
+            for (int64_t off = (int64_t)threadIdx.x * 16; off < row_bytes; off += kExpandChunk) expand_store16(dst + off, u32x4{0u, 0u, 0u, 0u});
+            if (x_sf)
+                for (int j = threadIdx.x; j < sf_cols; j += kThreads) out_sf[sf_col_major ? (int64_t)j * out_sf_ld + r : (int64_t)r * out_sf_ld + j] = 0u;
+        }
     }
 }
 
@@ -319,11 +322,14 @@ extern "C" int tk_expand_to_fused(const void *x, int64_t num_tokens, int64_t row
     if (rc != TK_OK) return rc;
     const int64_t chunks = (row_bytes + kExpandChunk - 1) / kExpandChunk;
     const int64_t copy_blocks = (num_tokens + 7) / 8 * 8 * num_topk * chunks;
-    const int64_t grid = copy_blocks + num_expanded;
+    // padding workgroups take 8 KB of consecutive rows each, two stores per thread.  Measured (us per call, 1 / 2 / 4
+    // rows per workgroup): 8 KB rows 64.4 / 69.7 / 71.0; 4 KB rows with scales 41.4 / 36.0 / 37.0
+    const int pad_rows = row_bytes >= 8192 ? 1 : (int)(8192 / row_bytes > 8 ? 8 : 8192 / row_bytes);
+    const int64_t grid = copy_blocks + (num_expanded + pad_rows - 1) / pad_rows;
     if (grid == 0) return TK_OK;
     hipLaunchKernelGGL(expand_to_fused_kernel, dim3((unsigned)grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint8_t *>(x), row_bytes, token_topk_to_pos, num_topk, (int)chunks, (int)copy_blocks,
                        (int)num_tokens, (int)num_expanded, static_cast<uint8_t *>(out), pos_to_expert,
-                       static_cast<const uint32_t *>(x_sf), sf_cols, static_cast<uint32_t *>(out_sf), out_sf_ld, sf_col_major);
+                       static_cast<const uint32_t *>(x_sf), sf_cols, static_cast<uint32_t *>(out_sf), out_sf_ld, sf_col_major, pad_rows);
     return (int)hipGetLastError();
 }
