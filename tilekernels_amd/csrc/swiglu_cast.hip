@@ -3,8 +3,8 @@
 // x[R, 2H]: gate = columns [0, H), up = columns [H, 2H).  The activation never touches HBM: a lane
 // loads 8 gate and 8 up values (two 16-byte loads for bf16), computes v = g/(1+exp(-g))*u in fp32,
 // and the 16 lanes that share a 128-column group reduce |v| with DPP, derive the scale and
-// convert straight to packed FP8.  Tiling is the one of the per-token cast: 16 rows x 512 output
-// columns per workgroup, 4 rows per wave, all eight loads of a lane in flight before first use.
+// convert straight to packed FP8.  A wave holds four 512-column pieces (of one row, or of four rows:
+// see the tile shapes below), all eight loads of a lane in flight before first use.
 // Padding rows (pos_to_expert < 0) are not read; zeros are written for their codes and scales.
 //
 // Reference semantics: tile_kernels/quant/swiglu_forward_and_per_token_cast_kernel.py:61-170,
@@ -85,27 +85,34 @@ __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
     return (pos >= 0 && pos < p.num_weights) ? uniform_load(p.topk_weights + pos) : 0.0f;
 }
 
-// Tile shapes as in the per-token cast (RPW = rows per wave):
-//   WIDE  (row-major scales):     RPW rows x (W*512) output columns, W = blockDim.x/64 waves side by side; the tile's
-//         scales are RPW contiguous runs of 16, staged in LDS and stored as whole segments
-//   !WIDE (column-major layouts): 4*RPW rows x 512 columns, the 4 waves stacked, scales stored transposed
-// FULL: the tile grid covers the matrix exactly: no bounds checks are compiled in.
+// Tile shapes (a wave always holds RPW pieces of 512 output columns, each with its gate and its up half):
+//   T_ROW     (row-major scales, H a multiple of RPW*512): W rows x (RPW*512) columns, one row per wave.  The RPW*4
+//             scales a wave produces are neighbours in the scale row, so the wave stores them itself as one
+//             contiguous run: no LDS stage and no workgroup barrier at the end of the tile
+//   T_WIDE    (row-major scales, other H): RPW rows x (W*512) columns, W waves side by side; the tile's scales are
+//             RPW contiguous runs, staged in LDS and stored as whole segments
+//   T_STACKED (column-major layouts): 4*RPW rows x 512 columns, the 4 waves stacked, scales stored transposed
+// W = blockDim.x / 64.  FULL: the tile grid covers the matrix exactly: no bounds checks are compiled in.
 // MASK: pos_to_expert is given.
-template <typename InT, int CLAMP, int RPW, bool WIDE, bool FULL, bool MASK>
-__global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
+enum { T_STACKED = 0, T_WIDE = 1, T_ROW = 2 };
+
+template <typename InT, int CLAMP, int RPW, int TILE, bool FULL, bool MASK>
+__global__ __launch_bounds__(TILE != T_STACKED ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
     TK_SWIGLU_KERNEL_UNPACK;
+    constexpr bool WIDE = TILE == T_WIDE, ROW = TILE == T_ROW;
     constexpr int GPS = kStripCols / 128;   // 4 groups per strip
-    constexpr int ROWS = WIDE ? RPW : kWaves * RPW;
+    constexpr int ROWS = WIDE ? RPW : kWaves * RPW;          // rows per tile (T_ROW: blockDim.x / 64, not used as a constant)
     constexpr int SGPR = WIDE ? kMaxWideWaves * GPS : GPS;   // staged groups per row (capacity)
     // The counting variant loops over tiles (its grid is capped so that few workgroups touch the global
     // counters); every other variant has one workgroup per tile on a 2-D grid, which keeps integer
     // divisions and further kernel-argument loads out of the path to the first memory load.
     constexpr bool LOOP = CLAMP == 2;
-    const int nwaves = WIDE ? p.nwaves : kWaves;
+    const int nwaves = TILE != T_STACKED ? p.nwaves : kWaves;
+    const int rows = ROW ? nwaves : ROWS;
     using RS = RowScales<448, RPW, 16>;
-    __shared__ uint32_t stage[ROWS][SGPR];
+    __shared__ uint32_t stage[ROW ? 1 : ROWS][ROW ? 1 : SGPR];
 
-    const int total = LOOP ? ((p.R + ROWS - 1) / ROWS) * p.tiles_k : 1;
+    const int total = LOOP ? ((p.R + rows - 1) / rows) * p.tiles_k : 1;
     const int lane = threadIdx.x & 63, wave = wave_id();
     const bool has_weight = p.pos_to_token_topk != nullptr;
     const int own = lane & 15;
@@ -115,11 +122,12 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_c
     for (int tile = LOOP ? (int)blockIdx.x : 0; tile < total; tile += LOOP ? (int)gridDim.x : 1) {
         const int tile_m = LOOP ? tile / p.tiles_k : (int)blockIdx.x;
         const int tile_k = LOOP ? tile - tile_m * p.tiles_k : (int)blockIdx.y;
-        const int strip = WIDE ? tile_k * nwaves + wave : tile_k;
+        // piece r of the wave: row `row0 + (ROW ? 0 : r)`, columns from `col + (ROW ? r * 512 : 0)`
+        const int strip = ROW ? tile_k * RPW : (WIDE ? tile_k * nwaves + wave : tile_k);
         const int col = strip * kStripCols + lane * 8;
-        const bool col_ok = FULL || col < p.H;
-        const int row0 = tile_m * ROWS + srow;
+        const int row0 = ROW ? tile_m * nwaves + wave : tile_m * ROWS + srow;
         const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * (2 * (int64_t)p.H) + col;
+        constexpr int kRowStep = ROW ? 0 : 1, kColStep = ROW ? kStripCols : 0;
 
         TK_TRACE(0);
         Raw8<InT> rg[RPW], ru[RPW];
@@ -128,13 +136,15 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_c
         // round trip in front of the loads instead of one per row
         int expert[RPW];
 #pragma unroll
-        for (int r = 0; r < RPW; ++r) expert[r] = (MASK && (FULL || row0 + r < p.R)) ? uniform_load(p.pos_to_expert + row0 + r) : 0;
-        if constexpr (MASK && RPW == 4)   // all four values must exist here, so their loads are issued together above
+        for (int r = 0; r < RPW; ++r)
+            expert[r] = (MASK && (FULL || row0 + r * kRowStep < p.R)) ? uniform_load(p.pos_to_expert + row0 + r * kRowStep) : 0;
+        if constexpr (MASK && RPW == 4 && !ROW)   // all four values must exist here, so their loads are issued together above
             asm volatile("" ::"s"(expert[0]), "s"(expert[1]), "s"(expert[2]), "s"(expert[3]));
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
-            live[r] = (FULL || row0 + r < p.R) && expert[r] >= 0;
-            const InT *xr = x + (int64_t)r * (2 * (int64_t)p.H);
+            live[r] = (FULL || row0 + r * kRowStep < p.R) && expert[r] >= 0;
+            const InT *xr = x + (int64_t)(r * kRowStep) * (2 * (int64_t)p.H) + r * kColStep;
+            const bool piece_ok = FULL || col + r * kColStep < p.H;
             if (FULL && !MASK) {
                 rg[r].load(xr);
                 ru[r].load(xr + p.H);
@@ -147,8 +157,8 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_c
                 ru[r].load(live[r] ? xr + p.H : src);
                 if (!live[r]) { rg[r].zero(); ru[r].zero(); }
             } else {
-                rg[r].load(xr, live[r] && col_ok);
-                ru[r].load(xr + p.H, live[r] && col_ok);
+                rg[r].load(xr, live[r] && piece_ok);
+                ru[r].load(xr + p.H, live[r] && piece_ok);
             }
         }
 
@@ -166,7 +176,7 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_c
                 v[r][i] = silu_mul<InT>(g[i], u[i]);
             }
             if (has_weight) {
-                const float w = live[r] ? row_weight(p, row0 + r) : 0.0f;
+                const float w = live[r] ? row_weight(p, row0 + r * kRowStep) : 0.0f;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) v[r][i] = v[r][i] * w;
             }
@@ -190,22 +200,32 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void swiglu_c
 #pragma unroll
             for (int r = 0; r < RPW; ++r) rs.inv[r] = live[r] ? rs.inv[r] : 0.0f;
         }
-        // lane j (< A) of a group computed the scale of row c*A + j
+        // lane j (< A) of a group computed the scale of piece c*A + j
         if (own < RS::A) {
 #pragma unroll
-            for (int c = 0; c < RS::NC; ++c)
-                stage[srow + c * RS::A + own][(WIDE ? wave * GPS : 0) + (lane >> 4)] =
-                    p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
+            for (int c = 0; c < RS::NC; ++c) {
+                if constexpr (ROW) {
+                    // group (lane >> 4) of piece c*A + own: the wave's scales form one run of RPW * 4 floats
+                    const int k = (strip + c * RS::A + own) * GPS + (lane >> 4);
+                    if (FULL || (row0 < p.R && k < p.sf.nk))
+                        st_stream4(reinterpret_cast<float *>(p.sf.base) + (int64_t)row0 * p.sf.ld + k, f2u(rs.own[c].sf));
+                } else {
+                    stage[srow + c * RS::A + own][(WIDE ? wave * GPS : 0) + (lane >> 4)] =
+                        p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
+                }
+            }
         }
 #pragma unroll
         for (int r = 0; r < RPW; ++r)
-            if (col_ok && (FULL || row0 + r < p.R))
-                quantise_store8<TK_E4M3, false>(v[r], rs.inv[r], p.out + (int64_t)(row0 + r) * p.H, col);
+            if ((FULL || col + r * kColStep < p.H) && (FULL || row0 + r * kRowStep < p.R))
+                quantise_store8<TK_E4M3, false>(v[r], rs.inv[r], p.out + (int64_t)(row0 + r * kRowStep) * p.H, col + r * kColStep);
         TK_TRACE(2);
-        __syncthreads();
-        if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
-        else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
-        if (LOOP && (int)gridDim.x < total) __syncthreads();   // stage is reused by the next tile
+        if constexpr (!ROW) {
+            __syncthreads();
+            if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
+            else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
+            if (LOOP && (int)gridDim.x < total) __syncthreads();   // stage is reused by the next tile
+        }
     }
     counter.flush(p.clamped_count);
 }
@@ -265,19 +285,20 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KER
     counter.flush(p.clamped_count);
 }
 
-// Rows per wave of the tiled kernel.  Measured on MI355X at [8192, 4096] bf16 (us per call, row-major
-// scales): 1 row 16.5, 2 rows 15.7, 4 rows 15.0.
+// Pieces per wave of the tiled kernel.  Measured on MI355X at [8192, 4096] bf16 (us per call, row-major
+// scales, pieces = rows): 1 row 16.5, 2 rows 15.7, 4 rows 15.0.  With the four pieces taken from one row
+// (T_ROW) instead of four rows (T_WIDE): 14.75 -> 14.63.
 #ifndef TK_SWIGLU_RPW
 #define TK_SWIGLU_RPW 4
 #endif
 constexpr int kSwigluRowsPerWave = TK_SWIGLU_RPW;
 
-template <typename InT, int CLAMP, int RPW, bool WIDE>
+template <typename InT, int CLAMP, int RPW, int TILE>
 static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t stream) {
     const int strips = (p.H + kStripCols - 1) / kStripCols;
-    const int waves = WIDE ? wide_tile_waves(strips) : kWaves;
-    const int rows = WIDE ? RPW : kWaves * RPW;
-    const int cols = WIDE ? waves * kStripCols : kStripCols;
+    const int waves = TILE == T_WIDE ? wide_tile_waves(strips) : kWaves;
+    const int rows = TILE == T_WIDE ? RPW : (TILE == T_ROW ? waves : kWaves * RPW);
+    const int cols = TILE == T_WIDE ? waves * kStripCols : (TILE == T_ROW ? RPW * kStripCols : kStripCols);
     const int tiles_m = (p.R + rows - 1) / rows;
     p.tiles_k = (p.H + cols - 1) / cols;
     p.nwaves = waves;
@@ -287,11 +308,11 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
                                  : dim3((unsigned)tiles_m, (unsigned)p.tiles_k);
     const bool full = p.R % rows == 0 && p.H % cols == 0;
     if (p.pos_to_expert) {
-        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, true, true>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
-        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, false, true>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, true, true>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, false, true>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
     } else {
-        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, true, false>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
-        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, WIDE, false, false>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, true, false>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, false, false>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
     }
 }
 
@@ -300,9 +321,12 @@ static hipError_t launch_swiglu_2(SwigluParams &p, bool row_group, int max_block
     if (row_group) {
         const int grid = max_blocks > 0 && max_blocks < p.R ? max_blocks : p.R;
         hipLaunchKernelGGL((swiglu_rowgroup_kernel<InT, CLAMP>), dim3(grid), dim3(kThreads), 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+    } else if (p.sf.layout != TK_SF_ROW_F32) {
+        launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, T_STACKED>(p, max_blocks, stream);
+    } else if (p.H % (kSwigluRowsPerWave * kStripCols) == 0) {
+        launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, T_ROW>(p, max_blocks, stream);
     } else {
-        if (p.sf.layout == TK_SF_ROW_F32) launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, true>(p, max_blocks, stream);
-        else launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, false>(p, max_blocks, stream);
+        launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, T_WIDE>(p, max_blocks, stream);
     }
     return hipGetLastError();
 }
