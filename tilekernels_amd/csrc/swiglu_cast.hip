@@ -296,7 +296,10 @@ constexpr int kSwigluRowsPerWave = TK_SWIGLU_RPW;
 template <typename InT, int CLAMP, int RPW, int TILE>
 static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t stream) {
     const int strips = (p.H + kStripCols - 1) / kStripCols;
-    const int waves = TILE == T_WIDE ? wide_tile_waves(strips) : kWaves;
+    // T_ROW, rows per workgroup (= waves), us per call at [8192, 4096] dense / [48128, 4096] with a third of the rows
+    // masked: 1: 14.9 / 61.6, 2: 14.85 / 62.1, 4: 14.68 / 62.9, 8: 15.15 / 63.4.  A masked batch is better off with
+    // single-wave workgroups: a wave whose row is padding is done at once and frees its slot alone.
+    const int waves = TILE == T_WIDE ? wide_tile_waves(strips) : (TILE == T_ROW && p.pos_to_expert ? 1 : kWaves);
     const int rows = TILE == T_WIDE ? RPW : (TILE == T_ROW ? waves : kWaves * RPW);
     const int cols = TILE == T_WIDE ? waves * kStripCols : (TILE == T_ROW ? RPW * kStripCols : kStripCols);
     const int tiles_m = (p.R + rows - 1) / rows;
