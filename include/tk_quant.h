@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define TK_QUANT_VERSION 105 /* major*10000 + minor*100 + patch */
+#define TK_QUANT_VERSION 106 /* major*10000 + minor*100 + patch */
 
 enum tk_dtype { TK_BF16 = 0, TK_F32 = 1 };
 enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1 };
@@ -178,7 +178,8 @@ int tk_check_swiglu_backward_per_token_cast(const void *x, const float *x_sf, in
 /*
  * Per-channel cast: E4M3 with one scale per `num_per_tokens` (32 or 128) tokens x 1 column, scales fp32
  * row-major out_sf[ceil(M / num_per_tokens), K].  The input is
- *   x_sf == NULL, swiglu == 0 : bf16 x[num_tokens, K]
+ *   x_sf == NULL, swiglu == 0 : bf16 x[num_tokens, K]; fp32 too when transpose == 0 (the reference's
+ *                               transposing and SwiGLU forms take bf16 only)
  *   x_sf != NULL              : E4M3 codes x[num_tokens, K] with fp32 scales x_sf[num_tokens, K / 128]
  *                               (1 x 128 groups); every element is first dequantised, code * scale
  *   swiglu != 0               : bf16 x[num_tokens, 2K]; the value cast is bf16(g / (1 + exp(-g)) * u) with

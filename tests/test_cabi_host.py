@@ -168,7 +168,12 @@ def test_per_channel_cast_validation(lib):
     assert check_pc(lib) == OK
     assert check_pc(lib, npt=32, tr=1) == OK
     assert check_pc(lib, npt=64) == GROUP
-    assert check_pc(lib, dt=1) == DTYPE                                 # bf16 (or FP8 + scales) only
+    assert check_pc(lib, dt=1) == OK                                    # fp32: plain and gathered casts only
+    assert check_pc(lib, dt=1, T=128, p2t=P) == OK
+    assert check_pc(lib, dt=1, tr=1) == DTYPE
+    assert check_pc(lib, dt=1, sw=1) == DTYPE
+    assert check_pc(lib, dt=1, x_sf=P, K=256) == DTYPE
+    assert check_pc(lib, dt=2) == DTYPE
     assert check_pc(lib, M=250) == SHAPE                                # M % 16
     assert check_pc(lib, K=20) == SHAPE                                 # K % 8
     assert check_pc(lib, T=128) == SHAPE                                # without a gather the input must hold M rows

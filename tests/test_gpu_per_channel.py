@@ -82,6 +82,31 @@ def test_per_channel_cast_and_transpose(num_tokens, hidden, num_per_tokens, roun
     assert_same(got[1], want[1], 'scales')
 
 
+@pytest.mark.parametrize('round_sf', [False, True])
+@pytest.mark.parametrize('hidden', [256, 2048, 7168])
+@pytest.mark.parametrize('moe', [None, (513, 2, 9, 16)])
+def test_per_channel_cast_fused_fp32_input(moe, hidden, round_sf):
+    """fp32 input (tile_kernels/quant/common.py:84-88 admits it for the plain and the gathered cast)."""
+    tk = _tk()
+    if moe is None:
+        g = torch.Generator().manual_seed(hidden + 1)
+        x, pos = torch.randn((1024, hidden), generator=g), None
+    else:
+        T, K, E, alignment = moe
+        x, pos = _moe_case(T, K, E, hidden, seed=hidden + T + 1, alignment=alignment)
+        x = torch.randn(x.shape, generator=torch.Generator().manual_seed(hidden))      # full fp32 mantissas
+    x[3, 5] = 3.0e38
+    want = torch_ref.per_channel_cast_fused(x, 128, None, round_sf, pos)
+    got = tk.quant.per_channel_cast_fused(x.cuda(), 'e4m3', num_per_tokens=128, round_sf=round_sf,
+                                          pos_to_token=None if pos is None else pos.cuda())
+    assert_same(got[0], want[0], 'codes')
+    assert_same(got[1], want[1], 'scales')
+    if moe is None:
+        got = tk.quant.per_channel_cast(x.cuda(), 'e4m3', 128, round_sf)
+        assert_same(got[0], want[0], 'codes')
+        assert_same(got[1], want[1], 'scales')
+
+
 def check_swiglu_per_channel(got, want, npt, round_sf, transposed, what=''):
     codes, sf = got
     codes_ref, sf_ref = want

@@ -40,7 +40,7 @@ constexpr int kPcThreads = 32 * kPcParts;                // 512
 // the reader still takes 16 bytes at a time.
 constexpr int kPcPitch = kPcTileM + 16;
 
-enum { PC_BF16 = 0, PC_E4M3 = 1, PC_SWIGLU = 2 };
+enum { PC_BF16 = 0, PC_E4M3 = 1, PC_SWIGLU = 2, PC_F32 = 3 };
 
 struct PerChannelParams {
     const void *x;
@@ -64,6 +64,13 @@ struct PerChannelParams {
 
 template <int MODE> struct PcRaw { typedef Raw8<bf16_t> type; };
 template <> struct PcRaw<PC_E4M3> { typedef Raw8<e4m3in_t> type; };
+template <> struct PcRaw<PC_F32> { typedef Raw8<float> type; };
+
+// Makes the compiler treat the packed input as redefined here, so that what was unpacked from it before
+// cannot be kept alive across this point.
+__device__ __forceinline__ void forget_unpacked(Raw8<bf16_t> &r) { asm volatile("" : "+v"(r.w)); }
+__device__ __forceinline__ void forget_unpacked(Raw8<e4m3in_t> &r) { asm volatile("" : "+v"(r.w)); }
+__device__ __forceinline__ void forget_unpacked(Raw8<float> &) {}   // nothing is unpacked: the registers are the values
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{a, b}), bf16x2));
@@ -155,6 +162,9 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
                     raw[r].load(reinterpret_cast<const uint8_t *>(p.x) + (int64_t)src * in_ld + col);
                     raw[r].s = p.x_sf[(int64_t)src * (p.K >> 7) + (col >> 7)];
                     if (GATHER && !valid) raw[r].zero();
+                } else if constexpr (MODE == PC_F32) {
+                    raw[r].load(reinterpret_cast<const float *>(p.x) + (int64_t)src * in_ld + col);
+                    if (GATHER && !valid) raw[r].zero();
                 } else {
                     raw[r].load(reinterpret_cast<const uint16_t *>(p.x) + (int64_t)src * in_ld + col);
                     if (GATHER && !valid) raw[r].zero();
@@ -177,7 +187,7 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
     // the tile is unpacked a second time after the scales are known; without this the compiler keeps
     // all 64 unpacked values alive across the two barriers instead
 #pragma unroll
-    for (int r = 0; r < kPcRows; ++r) asm volatile("" : "+v"(raw[r].w));
+    for (int r = 0; r < kPcRows; ++r) forget_unpacked(raw[r]);
     {
         u32x4 *dst = reinterpret_cast<u32x4 *>(&part[wave * 2 + half][hl * 8]);
         dst[0] = u32x4{f2u(m[0]), f2u(m[1]), f2u(m[2]), f2u(m[3])};
@@ -270,6 +280,9 @@ static void launch_per_channel_2(const PerChannelParams &p, bool transpose, hipS
     if constexpr (MODE == PC_SWIGLU) {
         if (transpose) TK_PC_LAUNCH(true, false);
         else TK_PC_LAUNCH(false, false);
+    } else if constexpr (MODE == PC_F32) {   // checked before: no transposed output from fp32
+        if (p.pos_to_token) TK_PC_LAUNCH(false, true);
+        else TK_PC_LAUNCH(false, false);
     } else if (p.pos_to_token) {
         if (transpose) TK_PC_LAUNCH(true, true);
         else TK_PC_LAUNCH(false, true);
@@ -298,7 +311,8 @@ extern "C" int tk_check_per_channel_cast(const void *x, int x_dtype, const float
     (void)round_sf;
     (void)pos_to_token;
     (void)transpose;
-    if (x_dtype != TK_BF16) return TK_ERR_BAD_DTYPE;
+    if (x_dtype != TK_BF16 && x_dtype != TK_F32) return TK_ERR_BAD_DTYPE;
+    if (x_dtype == TK_F32 && (x_sf || swiglu || transpose)) return TK_ERR_BAD_DTYPE;   // as the reference: plain and gathered casts only
     if (num_per_tokens != 32 && num_per_tokens != 128) return TK_ERR_BAD_GROUP;
     if (num_tokens < 0 || M < 0 || K <= 0 || K % 8 != 0 || M % 16 != 0) return TK_ERR_BAD_SHAPE;
     if (x_sf && (K % 128 != 0 || swiglu)) return TK_ERR_BAD_MODE;
@@ -338,6 +352,7 @@ extern "C" int tk_per_channel_cast(const void *x, int x_dtype, const float *x_sf
     hipError_t e;
     if (swiglu) e = launch_per_channel<PC_SWIGLU>(p, num_per_tokens, transpose != 0, s);
     else if (x_sf) e = launch_per_channel<PC_E4M3>(p, num_per_tokens, transpose != 0, s);
+    else if (x_dtype == TK_F32) e = launch_per_channel<PC_F32>(p, num_per_tokens, false, s);
     else e = launch_per_channel<PC_BF16>(p, num_per_tokens, transpose != 0, s);
     return (int)e;
 }

@@ -23,7 +23,7 @@ def _launch(x, x_sf, num_tokens, hidden, pos_to_token, num_tokens_out, num_per_t
     if num_tokens_out > 0:
         with torch.cuda.device(dev):
             rc = lib.tk_per_channel_cast(
-                x.data_ptr(), _ffi.TK_BF16, _ffi.ptr(x_sf), num_tokens, hidden, _ffi.ptr(pos_to_token), num_tokens_out,
+                x.data_ptr(), _ffi.TK_F32 if x.dtype == torch.float32 else _ffi.TK_BF16, _ffi.ptr(x_sf), num_tokens, hidden, _ffi.ptr(pos_to_token), num_tokens_out,
                 out.data_ptr(), out_sf.data_ptr(), num_per_tokens, int(round_sf), int(transpose), int(swiglu),
                 int(swiglu_clamp_value is not None), 0.0 if swiglu_clamp_value is None else float(swiglu_clamp_value),
                 _ffi.current_stream(dev))
@@ -69,8 +69,8 @@ def per_channel_cast_fused(
         assert x.dtype == torch.float8_e4m3fn
         assert x_sf.dim() == 2 and x_sf.is_contiguous() and x_sf.dtype == torch.float32
         assert x_sf.size(0) == num_tokens and x_sf.size(1) * 128 == hidden
-    elif x.dtype != torch.bfloat16:
-        raise NotImplementedError('per-channel casts take bf16 (or FP8 with scales) input')
+    else:
+        assert x.dtype in (torch.bfloat16, torch.float32)
     assert hidden % 8 == 0
 
     return _launch(x, x_sf, num_tokens, hidden, pos_to_token, num_tokens_out, num_per_tokens, round_sf, False)
