@@ -312,7 +312,44 @@ def op_swiglu_weighted():
     return launch, algo, nbytes(x, out, sf), cpu
 
 
+def op_e5m6(direction):
+    """per_token_cast(fmt='e5m6') of bf16 [8192, 4096] (one scale per row) and its dequantisation."""
+    def build():
+        import tilekernels_amd as tk
+        from tilekernels_amd import _ffi
+        lib = _ffi.load()
+        M, K = 8192, 4096
+        x = torch.randn((M, K), device='cuda', dtype=torch.bfloat16)
+        codes = torch.empty((M, K * 3 // 2), device='cuda', dtype=torch.uint8)
+        sf = torch.empty((M, 1), device='cuda', dtype=torch.float32)
+        back = torch.empty((M, K), device='cuda', dtype=torch.bfloat16)
+        stream = _ffi.current_stream(x.device)
+
+        def cast():
+            rc = lib.tk_per_token_cast(x.data_ptr(), _ffi.TK_BF16, M, K, K, codes.data_ptr(), sf.data_ptr(), 1, _ffi.TK_E5M6, K,
+                                       _ffi.TK_SF_ROW_F32, 1, _ffi.TK_CAST_AND_SF, stream)
+            assert rc == 0, rc
+        def uncast():
+            rc = lib.tk_cast_back(codes.data_ptr(), _ffi.TK_E5M6, M, K, sf.data_ptr(), 1, _ffi.TK_SF_ROW_F32, 1, K, back.data_ptr(),
+                                  _ffi.TK_BF16, stream)
+            assert rc == 0, rc
+        cast()
+        ts = [x, codes, sf] if direction == 'cast' else [codes, sf, back]
+
+        def cpu():
+            from oracle import torch_ref
+            if direction == 'cast':
+                xc = x.cpu()
+                return lambda: torch_ref.cast_to_e5m6(xc, K, round_sf=True)
+            xq = (codes.cpu(), sf.cpu())
+            return lambda: torch_ref.cast_back_from_e5m6(xq, 'bf16', (1, K))
+        return (cast if direction == 'cast' else uncast), nbytes(*ts), nbytes(x, codes, sf, back), cpu
+    return build
+
+
 OPS = [
+    Op('per_token_cast_e5m6', "per_token_cast fmt='e5m6' (12-bit, one scale per row) round_sf, bf16 [8192,4096]", op_e5m6('cast')),
+    Op('cast_back_e5m6', 'cast_back of e5m6 -> bf16, [8192,4096]', op_e5m6('back')),
     Op('per_token_cast_with_sf_only', 'per_token_cast_with_sf_only e4m3 1x128, bf16 [4096,7168]', op_cast_variant('token', 'sf_only')),
     Op('per_token_cast_with_precomputed_sf', 'per_token_cast_with_precomputed_sf e4m3 1x128, bf16 [4096,7168]',
        op_cast_variant('token', 'given_sf')),

@@ -37,10 +37,10 @@
 extern "C" {
 #endif
 
-#define TK_QUANT_VERSION 106 /* major*10000 + minor*100 + patch */
+#define TK_QUANT_VERSION 107 /* major*10000 + minor*100 + patch */
 
 enum tk_dtype { TK_BF16 = 0, TK_F32 = 1 };
-enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1 };
+enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1, TK_E5M6 = 2 };
 enum tk_sf_layout { TK_SF_ROW_F32 = 0, TK_SF_COL_F32 = 1, TK_SF_COL_UE8M0 = 2 };
 enum tk_mode {
     TK_CAST_AND_SF = 0, /* write codes and scales                                  */
@@ -76,6 +76,13 @@ enum tk_status {
  *   out          E4M3: M*K bytes;  E2M1: M*K/2 bytes, element 2t in the low nibble of byte t
  *   group        16, 32, 64, 128, or K (one scale per row; needs K % 64 == 0 and TK_CAST_AND_SF)
  *   requirements K % 8 == 0; x and x_row_stride 16-byte aligned; out 8-byte aligned
+ *
+ * fmt = TK_E5M6 (tile_kernels/quant/per_token_cast_to_e5m6_kernel.py:10-70, 172-215): a 12-bit float, the top
+ * 12 bits of an IEEE fp16 (sign, 5 exponent bits, 6 mantissa bits), QMAX = 65024, floor = 1e-4, one scale per
+ * row (group == K, any K % 8 == 0, TK_CAST_AND_SF only).  code = the fp16 of x * inv rounded toward zero, cut
+ * to 12 bits and incremented when (kept lsb) + (low 17 bits of the fp32 pattern of x * inv) > 0x10000: round
+ * to nearest even for |x * inv| >= 2^-14.  out: M * K * 3/2 bytes; codes c0..c7 of eight consecutive elements
+ * form a 96-bit string, c0 in the most significant bits, stored as three 32-bit words, high word first.
  */
 int tk_per_token_cast(const void *x, int x_dtype, int64_t M, int64_t K, int64_t x_row_stride, void *out,
                       void *sf, int64_t sf_ld, int fmt, int group, int sf_layout, int round_sf, int mode,
@@ -203,11 +210,12 @@ int tk_check_per_channel_cast(const void *x, int x_dtype, const float *x_sf, int
 
 /*
  * Dequantisation: out[m, k] = float(code[m, k]) * sf[m / bm, k / bk] (one fp32 product), stored as
- * fp32 or rounded to bf16 (nearest even).  x: E4M3 bytes [M, K] or packed E2M1 bytes [M, K/2],
- * contiguous (K in logical elements); x_sf in any of the three layouts.
+ * fp32 or rounded to bf16 (nearest even).  x: E4M3 bytes [M, K], packed E2M1 bytes [M, K/2] or packed E5M6
+ * words [M, K*3/2 bytes] (layout as written by tk_per_token_cast), contiguous (K in logical elements); x_sf in
+ * any of the three layouts.
  * Stands behind tile_kernels.quant.cast_back and per_token_cast_back
- * (tile_kernels/quant/cast_back_kernel.py:77-143).
- *   requirements K % 8 == 0, bk % 8 == 0; out 16-byte aligned; x 8-byte (E4M3) / 4-byte (E2M1) aligned
+ * (tile_kernels/quant/cast_back_kernel.py:77-143, cast_back_e5m6_kernel.py:12-41, 141-176).
+ *   requirements K % 8 == 0, bk % 8 == 0; out 16-byte aligned; x 8-byte (E4M3) / 4-byte (E2M1, E5M6) aligned
  */
 int tk_cast_back(const void *x, int x_fmt, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld, int x_sf_layout,
                  int bm, int bk, void *out, int out_dtype, void *stream);

@@ -9,6 +9,7 @@ pure-torch implementations:
 * ``per_channel_cast_fused``    <- tile_kernels/torch/per_channel_cast_fused.py:9-46
 * ``unpack_from_e2m1fn_x2``     <- tile_kernels/quant/common.py:247-295
 * ``encode_e2m1``               <- tile_kernels/torch/cast.py:224-252 (same result, closed form)
+* ``cast_to_e5m6`` / ``cast_back_from_e5m6`` <- tile_kernels/torch/cast_e5m6.py:145-258
 
 Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import
 it.  The shipped package never does: it has no CPU path at all.
@@ -33,6 +34,14 @@ How each function is pinned (all pins live in tests/test_oracle_*.py and run wit
 * ``swiglu_backward`` is checked against float64 autograd of ``silu(g) * u * w`` (a dropped term,
   a wrong sign or swapped halves fails it), against hand-set clamp cases, and its ``fma_f32`` helper
   against the C library's correctly rounded ``fmaf`` on operands built to hit double rounding.
+* the E5M6 pair: the fp32 -> fp16 round-toward-zero step against a brute-force "largest fp16 magnitude
+  not above |x|" search, the 12-bit rounding against an independent nearest-ties-to-even search over
+  all 4096 codes for values whose fp16 form is normal, the 96-bit packing against a Python big-integer
+  concatenation and hand-built words, the round trip through ``cast_back_from_e5m6``, and the
+  reference's three special inputs.  Below the smallest normal fp16 the reference does NOT round to
+  nearest (it rounds on bits of the fp32 pattern that are not the ones dropped; cast_e5m6.py:75-81,
+  per_token_cast_to_e5m6_kernel.py:49-56): that range is restated from those lines and covered only by
+  hand-computed cases, so parity with the reference is unpinned there beyond those cases.
 """
 from typing import Optional, Tuple, Union
 
@@ -44,6 +53,8 @@ E4M3_MAX = 448.0
 E2M1_MAX = 6.0
 E4M3_AMAX_FLOOR = 1e-4
 E2M1_AMAX_FLOOR = 6.0 * 2.0 ** -126
+E5M6_MAX = 65024.0            # (2 - 2^-6) * 2^15: the largest fp16 whose low four mantissa bits are zero
+E5M6_AMAX_FLOOR = 1e-4
 
 # magnitudes of the eight E2M1 codes, index = 3-bit code (exp:2 | mant:1)
 E2M1_VALUES = (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0)
@@ -548,3 +559,101 @@ def expand_to_fused_with_sf(x: QuantTensor, num_per_channels: int, token_topk_to
     keep = pos >= 0
     out_sf[pos[keep]] = sf[src[keep]]
     return out, out_sf
+
+
+# ------------------------------------------------------------------------------------------------
+# E5M6: a 12-bit float (sign, 5 exponent bits, 6 mantissa bits) = the top 12 bits of an IEEE fp16.
+# Eight codes are stored as three 32-bit words.
+
+def fp16_bits_toward_zero(x: torch.Tensor) -> torch.Tensor:
+    """fp32 -> the bit pattern (int32, 0..0xFFFF) of the fp16 nearest to zero-ward of it: finite values
+    beyond the fp16 range become infinity, NaNs 0x7FFF (tile_kernels/torch/cast_e5m6.py:37-62)."""
+    bits = x.contiguous().view(torch.int32)
+    mag = bits & 0x7FFFFFFF
+    e, m = mag >> 23, mag & 0x7FFFFF
+    sig = m | 0x800000                                          # significand with its leading one
+    out = torch.zeros_like(mag)
+    normal = (e >= 113) & (e <= 142)
+    out = torch.where(normal, ((e - 112) << 10) | (m >> 13), out)
+    sub = (e >= 103) & (e <= 112)                               # fp16 subnormals: 2^-24 .. 2^-14
+    out = torch.where(sub, sig >> (126 - e).clamp(0, 31), out)
+    out = torch.where(e > 142, torch.full_like(out, 0x7C00), out)
+    out = torch.where(mag > 0x7F800000, torch.full_like(out, 0x7FFF), out)
+    return out | ((bits >> 16) & 0x8000)
+
+
+def encode_e5m6(x: torch.Tensor) -> torch.Tensor:
+    """fp32 -> 12-bit E5M6 codes (int32).  The fp16 pattern is cut to 12 bits and bumped when
+    (kept lsb) + (low 17 bits of the fp32 pattern) exceeds 0x10000 (cast_e5m6.py:75-81): round to
+    nearest, ties to even, wherever the fp16 form is normal."""
+    bits = x.contiguous().view(torch.int32)
+    kept = fp16_bits_toward_zero(x) >> 4
+    bump = ((kept & 1) + (bits & 0x1FFFF)) > 0x10000
+    return (kept + bump.to(torch.int32)) & 0xFFF
+
+
+def pack_e5m6(codes: torch.Tensor) -> torch.Tensor:
+    """[M, K] codes -> uint8 [M, K * 3 // 2]: each 8 codes form a 96-bit string, first code in the
+    most significant bits, stored as three little-endian 32-bit words from the high word down
+    (cast_e5m6.py:83-101)."""
+    m, k = codes.shape
+    c = codes.to(torch.int64).view(m, k // 8, 8)
+    hi = (c[..., 0] << 36) | (c[..., 1] << 24) | (c[..., 2] << 12) | c[..., 3]      # 48 bits
+    lo = (c[..., 4] << 36) | (c[..., 5] << 24) | (c[..., 6] << 12) | c[..., 7]
+    words = torch.stack([hi >> 16, ((hi & 0xFFFF) << 16) | (lo >> 32), lo & 0xFFFFFFFF], dim=-1)
+    signed = torch.where(words >= 2 ** 31, words - 2 ** 32, words).to(torch.int32)
+    return signed.view(m, k // 8 * 3).view(torch.uint8)
+
+
+def unpack_e5m6(packed: torch.Tensor) -> torch.Tensor:
+    """uint8 [M, K * 3 // 2] -> int32 codes [M, K] (cast_e5m6.py:104-133)."""
+    m = packed.shape[0]
+    w = packed.contiguous().view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    w = w.view(m, w.shape[1] // 3, 3)
+    hi = (w[..., 0] << 16) | (w[..., 1] >> 16)
+    lo = ((w[..., 1] & 0xFFFF) << 32) | w[..., 2]
+    cols = [(hi >> 36) & 0xFFF, (hi >> 24) & 0xFFF, (hi >> 12) & 0xFFF, hi & 0xFFF,
+            (lo >> 36) & 0xFFF, (lo >> 24) & 0xFFF, (lo >> 12) & 0xFFF, lo & 0xFFF]
+    return torch.stack(cols, dim=-1).view(m, w.shape[1] * 8).to(torch.int32)
+
+
+def decode_e5m6(codes: torch.Tensor) -> torch.Tensor:
+    """12-bit codes -> fp32 values (the fp16 whose top 12 bits they are)."""
+    h = (codes.to(torch.int32) << 4) & 0xFFFF
+    h = torch.where(h >= 0x8000, h - 0x10000, h).to(torch.int16)
+    return h.view(torch.float16).to(torch.float32)
+
+
+def cast_to_e5m6(x: torch.Tensor, num_per_channels: int, use_tma_aligned_col_major_sf: bool = False,
+                 round_sf: bool = False, use_packed_ue8m0: bool = False) -> QuantTensor:
+    """Per-token E5M6 cast with one scale per ``num_per_channels`` channels (the reference's kernel
+    takes whole rows only): amax floored at 1e-4, scale = amax / 65024, multiplier 65024 / amax or,
+    with ``round_sf``, the inverse of the scale rounded up to a power of two
+    (tile_kernels/torch/cast_e5m6.py:145-222).  Returns ``(uint8 [M, K*3/2], scales)``."""
+    assert x.ndim == 2 and x.dtype in (torch.float32, torch.bfloat16)
+    xf = x.to(torch.float32)
+    h, w = xf.shape
+    assert w % num_per_channels == 0 and w % 8 == 0
+    amax = _block_amax(xf, 1, num_per_channels).clamp(min=E5M6_AMAX_FLOOR)
+    qmax = torch.full_like(amax, E5M6_MAX)
+    dq = amax / qmax
+    if round_sf:
+        bits = (dq.view(torch.int32) + 0x007FFFFF) & 0x7F800000
+        inv = ((254 - (bits >> 23)).clamp(min=0) << 23).view(torch.float32)      # 2^-(e-127), exactly
+    else:
+        bits = dq.view(torch.int32)
+        inv = qmax / amax
+    codes = encode_e5m6(xf * _expand_blocks(inv, 1, num_per_channels, h, w))
+    return pack_e5m6(codes), _format_sf(bits.contiguous(), use_tma_aligned_col_major_sf, use_packed_ue8m0)
+
+
+def cast_back_from_e5m6(x: QuantTensor, fmt: str, block_size: Tuple[int, int]) -> torch.Tensor:
+    """``(uint8 [M, K*3/2], scales)`` -> bf16 / fp32 [M, K]: code value times its block's scale, one
+    fp32 product (tile_kernels/torch/cast_e5m6.py:225-258)."""
+    packed, sf = x
+    assert packed.ndim == 2 and packed.dtype == torch.uint8 and fmt in ('bf16', 'fp32')
+    h, w = packed.shape[0], packed.shape[1] * 2 // 3
+    bh, bw = block_size
+    scales = _sf_as_fp32(sf)[:_ceil_div(h, bh), :_ceil_div(w, bw)]
+    out = decode_e5m6(unpack_e5m6(packed)) * _expand_blocks(scales, bh, bw, h, w)
+    return out.to(torch.float32 if fmt == 'fp32' else torch.bfloat16)

@@ -60,7 +60,12 @@ def test_per_token_cast_validation(lib):
     assert check_pt(lib) == OK
     assert check_pt(lib, M=0, x=0, out=0, sf=0) == OK                  # empty input: nothing to check
     assert check_pt(lib, dt=2) == DTYPE
-    assert check_pt(lib, fmt=2) == FMT
+    assert check_pt(lib, fmt=3) == FMT
+    assert check_pt(lib, fmt=2) == GROUP                               # E5M6: one scale per row only
+    assert check_pt(lib, fmt=2, K=1000, group=1000) == OK              # ... for any K % 8 == 0
+    assert check_pt(lib, fmt=2, K=1024, group=1024, layout=2, rnd=1) == OK
+    assert check_pt(lib, fmt=2, K=1024, group=1024, mode=1) == MODE
+    assert check_pt(lib, fmt=2, K=1024, group=1024, mode=2) == MODE
     assert check_pt(lib, mode=3) == MODE
     assert check_pt(lib, layout=3) == LAYOUT
     assert check_pt(lib, layout=2, rnd=0) == LAYOUT                    # UE8M0 bytes need power-of-two scales

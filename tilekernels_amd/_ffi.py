@@ -11,7 +11,7 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, 'lib', 'libtk_quant.so')
 
 TK_BF16, TK_F32 = 0, 1
-TK_E4M3, TK_E2M1 = 0, 1
+TK_E4M3, TK_E2M1, TK_E5M6 = 0, 1, 2
 TK_SF_ROW_F32, TK_SF_COL_F32, TK_SF_COL_UE8M0 = 0, 1, 2
 TK_CAST_AND_SF, TK_SF_ONLY, TK_CAST_GIVEN_SF = 0, 1, 2
 

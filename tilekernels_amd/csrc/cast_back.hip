@@ -96,7 +96,7 @@ using namespace tk;
 
 extern "C" int tk_check_cast_back(const void *x, int x_fmt, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld,
                                   int x_sf_layout, int bm, int bk, const void *out, int out_dtype) {
-    if (x_fmt != TK_E4M3 && x_fmt != TK_E2M1) return TK_ERR_BAD_FORMAT;
+    if (x_fmt != TK_E4M3 && x_fmt != TK_E2M1 && x_fmt != TK_E5M6) return TK_ERR_BAD_FORMAT;
     if (out_dtype != TK_BF16 && out_dtype != TK_F32) return TK_ERR_BAD_DTYPE;
     if (x_sf_layout < TK_SF_ROW_F32 || x_sf_layout > TK_SF_COL_UE8M0) return TK_ERR_BAD_LAYOUT;
     if (M < 0 || K <= 0 || K % 8 != 0) return TK_ERR_BAD_SHAPE;
@@ -104,7 +104,7 @@ extern "C" int tk_check_cast_back(const void *x, int x_fmt, int64_t M, int64_t K
     if (bm < 1 || bk < 8 || bk % 8 != 0) return TK_ERR_BAD_GROUP;
     if (M == 0) return TK_OK;
     if (!x || !x_sf || !out) return TK_ERR_NULL_POINTER;
-    if (!aligned_to(x, x_fmt == TK_E4M3 ? 8 : 4) || !aligned_to(out, 16)) return TK_ERR_MISALIGNED;
+    if (!aligned_to(x, x_fmt == TK_E4M3 ? 8 : 4) || !aligned_to(out, 16)) return TK_ERR_MISALIGNED;   // E5M6: 12-byte pieces of 4-byte words
     if (!aligned_to(x_sf, 4) || (x_sf_layout == TK_SF_COL_UE8M0 && x_sf_ld % 4 != 0)) return TK_ERR_MISALIGNED;
     const int64_t nm = (M + bm - 1) / bm, nk = (K + bk - 1) / bk;
     const int64_t need = x_sf_layout == TK_SF_ROW_F32 ? nk : (x_sf_layout == TK_SF_COL_F32 ? nm : 4 * nm);
@@ -123,8 +123,11 @@ extern "C" int tk_cast_back(const void *x, int x_fmt, int64_t M, int64_t K, cons
     if (x_fmt == TK_E4M3)
         e = out_dtype == TK_F32 ? launch_cast_back<e4m3in_t, true>(x, out, x_sf, x_sf_ld, (int)M, (int)K, x_sf_layout, bm, bk, s)
                                 : launch_cast_back<e4m3in_t, false>(x, out, x_sf, x_sf_ld, (int)M, (int)K, x_sf_layout, bm, bk, s);
-    else
+    else if (x_fmt == TK_E2M1)
         e = out_dtype == TK_F32 ? launch_cast_back<e2m1in_t, true>(x, out, x_sf, x_sf_ld, (int)M, (int)K, x_sf_layout, bm, bk, s)
                                 : launch_cast_back<e2m1in_t, false>(x, out, x_sf, x_sf_ld, (int)M, (int)K, x_sf_layout, bm, bk, s);
+    else
+        e = out_dtype == TK_F32 ? launch_cast_back<e5m6in_t, true>(x, out, x_sf, x_sf_ld, (int)M, (int)K, x_sf_layout, bm, bk, s)
+                                : launch_cast_back<e5m6in_t, false>(x, out, x_sf, x_sf_ld, (int)M, (int)K, x_sf_layout, bm, bk, s);
     return (int)e;
 }

@@ -134,22 +134,44 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
     }
 }
 
-// One scale per row (group == K): a workgroup per row, two passes over the row (the second one is
-// served by L2).  Reference: the `hidden == num_per_channels` branch,
-// tile_kernels/quant/per_token_cast_kernel.py:31-35.
-template <typename InT, int FMT>
+// One scale per row (group == K): a workgroup per row.  Rows of up to ITER * 2048 elements (ITER = 1..4) are held in
+// registers between the amax and the conversion, so they are read once; ITER == 0 takes longer rows in two passes (the
+// second one is served by L2).  Reference: the `hidden == num_per_channels` branch,
+// tile_kernels/quant/per_token_cast_kernel.py:31-35, and the E5M6 cast, which knows no other grouping
+// (per_token_cast_to_e5m6_kernel.py:88).
+template <int FMT> __host__ __device__ constexpr int64_t code_row_bytes(int64_t k) {
+    return FMT == TK_E4M3 ? k : (FMT == TK_E2M1 ? k / 2 : k / 8 * 12);
+}
+
+template <typename InT, int FMT, int ITER>
 __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERNEL_ARGS) {
     TK_PT_KERNEL_UNPACK;
     __shared__ uint32_t part[kThreads / 16];
     const int row = blockIdx.x;
     const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row * p.x_ld;   // plain (bf16 / fp32) inputs only
+    constexpr int N = ITER > 0 ? ITER : 1;
+    Raw8<InT> held[N];
     float amax = 0.0f;
-    for (int col = threadIdx.x * 8; col < p.K; col += kThreads * 8) {
-        Raw8<InT> raw;
-        raw.load_cached(x + col);
-        float v[8];
-        raw.get(v);
-        amax = __builtin_fmaxf(amax, absmax8(v));
+    if constexpr (ITER > 0) {
+#pragma unroll
+        for (int i = 0; i < ITER; ++i) {
+            const int col = (i * kThreads + threadIdx.x) * 8;
+            held[i].load(x + col, col < p.K);
+        }
+#pragma unroll
+        for (int i = 0; i < ITER; ++i) {
+            float v[8];
+            held[i].get(v);
+            amax = __builtin_fmaxf(amax, absmax8(v));
+        }
+    } else {
+        for (int col = threadIdx.x * 8; col < p.K; col += kThreads * 8) {
+            Raw8<InT> raw;
+            raw.load_cached(x + col);
+            float v[8];
+            raw.get(v);
+            amax = __builtin_fmaxf(amax, absmax8(v));
+        }
     }
     amax = group_allmax<16>(amax);
     if ((threadIdx.x & 15) == 0) part[threadIdx.x >> 4] = f2u(amax);
@@ -159,15 +181,39 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERN
     for (int i = 0; i < kThreads / 16; ++i) m = umax(m, part[i]);
     const Scale sc = make_scale<Fmt<FMT>::qmax>(u2f(m), Fmt<FMT>::floor_, p.round_sf != 0);
     if (threadIdx.x == 0) sf_store(p.sf, row, 0, sc);
-    const int64_t out_ld = FMT == TK_E4M3 ? p.K : p.K / 2;
-    uint8_t *out_row = p.out + (int64_t)row * out_ld;
-    for (int col = threadIdx.x * 8; col < p.K; col += kThreads * 8) {
-        Raw8<InT> raw;
-        raw.load(x + col);
-        float v[8];
-        raw.get(v);
-        quantise_store8<FMT, false>(v, sc.inv, out_row, col);
+    uint8_t *out_row = p.out + (int64_t)row * code_row_bytes<FMT>(p.K);
+    if constexpr (ITER > 0) {
+#pragma unroll
+        for (int i = 0; i < ITER; ++i) {
+            const int col = (i * kThreads + threadIdx.x) * 8;
+            float v[8];
+            held[i].get(v);
+            if (col < p.K) quantise_store8<FMT, false>(v, sc.inv, out_row, col);
+        }
+    } else {
+        for (int col = threadIdx.x * 8; col < p.K; col += kThreads * 8) {
+            Raw8<InT> raw;
+            raw.load(x + col);
+            float v[8];
+            raw.get(v);
+            quantise_store8<FMT, false>(v, sc.inv, out_row, col);
+        }
     }
+}
+
+template <typename InT, int FMT>
+static void launch_per_token_rowgroup(const PerTokenParams &p, hipStream_t stream) {
+    const int iters = (p.K + kThreads * 8 - 1) / (kThreads * 8);
+#define TK_ROWGROUP_LAUNCH(I) \
+    hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT, I>), dim3(p.M), dim3(kThreads), 0, stream, TK_PT_LAUNCH_ARGS(p))
+    switch (iters) {
+        case 1: TK_ROWGROUP_LAUNCH(1); break;
+        case 2: TK_ROWGROUP_LAUNCH(2); break;
+        case 3: TK_ROWGROUP_LAUNCH(3); break;
+        case 4: TK_ROWGROUP_LAUNCH(4); break;
+        default: TK_ROWGROUP_LAUNCH(0); break;
+    }
+#undef TK_ROWGROUP_LAUNCH
 }
 
 // Rows per wave.  Measured on MI355X (us per call): bf16 [4096, 7168] -> E4M3 1x128 row-major scales
@@ -206,7 +252,7 @@ template <typename InT, int FMT>
 static hipError_t launch_per_token(PerTokenParams &p, int group, hipStream_t stream) {
     if constexpr (!Elem<InT>::quantised) {
         if (group == p.K && group != 16 && group != 32 && group != 64 && group != 128) {
-            hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT>), dim3(p.M), dim3(kThreads), 0, stream, TK_PT_LAUNCH_ARGS(p));
+            launch_per_token_rowgroup<InT, FMT>(p, stream);
             return hipGetLastError();
         }
     }
@@ -227,14 +273,17 @@ extern "C" int tk_check_per_token_cast(const void *x, int x_dtype, int64_t M, in
                                        const void *out, const void *sf, int64_t sf_ld, int fmt, int group,
                                        int sf_layout, int round_sf, int mode) {
     if (x_dtype != TK_BF16 && x_dtype != TK_F32) return TK_ERR_BAD_DTYPE;
-    if (fmt != TK_E4M3 && fmt != TK_E2M1) return TK_ERR_BAD_FORMAT;
+    if (fmt != TK_E4M3 && fmt != TK_E2M1 && fmt != TK_E5M6) return TK_ERR_BAD_FORMAT;
     if (mode < TK_CAST_AND_SF || mode > TK_CAST_GIVEN_SF) return TK_ERR_BAD_MODE;
     if (sf_layout < TK_SF_ROW_F32 || sf_layout > TK_SF_COL_UE8M0) return TK_ERR_BAD_LAYOUT;
     if (sf_layout == TK_SF_COL_UE8M0 && !round_sf && mode != TK_CAST_GIVEN_SF) return TK_ERR_BAD_LAYOUT;
     if (M < 0 || K <= 0 || K % 8 != 0) return TK_ERR_BAD_SHAPE;
     if (M > INT32_MAX - 64 || K > INT32_MAX - 1024) return TK_ERR_TOO_LARGE;
-    const bool row_group = group == K && group != 16 && group != 32 && group != 64 && group != 128;
-    if (row_group) {
+    const bool row_group = fmt == TK_E5M6 || (group == K && group != 16 && group != 32 && group != 64 && group != 128);
+    if (fmt == TK_E5M6) {       // one scale per row, as the reference's kernel (per_token_cast_to_e5m6_kernel.py:88)
+        if (group != K) return TK_ERR_BAD_GROUP;
+        if (mode != TK_CAST_AND_SF) return TK_ERR_BAD_MODE;
+    } else if (row_group) {
         if (K % 64 != 0) return TK_ERR_BAD_GROUP;
         if (mode != TK_CAST_AND_SF) return TK_ERR_BAD_MODE;
     } else if (group != 16 && group != 32 && group != 64 && group != 128) {
@@ -277,6 +326,11 @@ extern "C" int tk_per_token_cast(const void *x, int x_dtype, int64_t M, int64_t 
     p.in_bm = p.in_bk = 1;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e;
+    if (fmt == TK_E5M6) {
+        if (x_dtype == TK_BF16) launch_per_token_rowgroup<bf16_t, TK_E5M6>(p, s);
+        else launch_per_token_rowgroup<float, TK_E5M6>(p, s);
+        return (int)hipGetLastError();
+    }
     if (x_dtype == TK_BF16)
         e = fmt == TK_E4M3 ? launch_per_token<bf16_t, TK_E4M3>(p, group, s) : launch_per_token<bf16_t, TK_E2M1>(p, group, s);
     else

@@ -26,10 +26,12 @@ inline int wide_tile_waves(int strips) {
 struct bf16_t { uint16_t bits; };
 struct e4m3in_t {};   // input that is itself E4M3 codes with block scales
 struct e2m1in_t {};   // input that is packed E2M1 codes (two per byte) with block scales
+struct e5m6in_t {};   // input that is packed E5M6 codes (eight per 12 bytes) with block scales
 
 template <typename T> struct Elem { static constexpr int bits = 8 * (int)sizeof(T); static constexpr bool quantised = false; };
 template <> struct Elem<e4m3in_t> { static constexpr int bits = 8; static constexpr bool quantised = true; };
 template <> struct Elem<e2m1in_t> { static constexpr int bits = 4; static constexpr bool quantised = true; };
+template <> struct Elem<e5m6in_t> { static constexpr int bits = 12; static constexpr bool quantised = true; };
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
@@ -40,6 +42,7 @@ template <typename T> __device__ __forceinline__ const void *elem_ptr(const void
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
 
 __device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
@@ -148,6 +151,33 @@ template <> struct Raw8<e2m1in_t> {
     }
 };
 
+// E5M6: a 12-bit float, the top 12 bits of an IEEE fp16 (sign, 5 exponent bits, 6 mantissa bits).  Eight
+// codes c0..c7 form a 96-bit string with c0 in the most significant bits, stored as three 32-bit words
+// from the high word down (reference: float_to_e5m6 / e5m6_to_float,
+// tile_kernels/quant/per_token_cast_to_e5m6_kernel.py:36-70, cast_back_e5m6_kernel.py:12-41).
+__device__ __forceinline__ float e5m6_value(uint32_t top12_in_bits_15_4) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(top12_in_bits_15_4 & 0xFFF0u));
+}
+template <> struct Raw8<e5m6in_t> {
+    u32x3 w;
+    float s;
+    __device__ __forceinline__ void load(const void *p) { w = __builtin_nontemporal_load(reinterpret_cast<const u32x3 *>(p)); }
+    __device__ __forceinline__ void load(const void *p, bool ok) {
+        w = u32x3{0u, 0u, 0u};
+        if (ok) load(p);
+    }
+    __device__ __forceinline__ void get(float (&v)[8]) const {
+        v[0] = e5m6_value(w.x >> 16) * s;
+        v[1] = e5m6_value(w.x >> 4) * s;
+        v[2] = e5m6_value((w.x << 8) | (w.y >> 24)) * s;
+        v[3] = e5m6_value(w.y >> 12) * s;
+        v[4] = e5m6_value(w.y) * s;
+        v[5] = e5m6_value((w.y << 12) | (w.z >> 20)) * s;
+        v[6] = e5m6_value(w.z >> 8) * s;
+        v[7] = e5m6_value(w.z << 4) * s;
+    }
+};
+
 __device__ __forceinline__ float absmax8(const float (&v)[8]) {
     float m = __builtin_fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1]));
 #pragma unroll
@@ -205,6 +235,7 @@ struct Scale {
 template <int QMAX> __device__ __forceinline__ float div_by_qmax(float a) {
     constexpr float c = (float)QMAX;
     constexpr float y = 1.0f / c;
+    if (QMAX != 448 && QMAX != 6) return a / c;   // E5M6 has one scale per row: the plain division costs nothing there
     if (a < 0x1p-100f) return a / c;
     const float q = a * y;
     return __builtin_fmaf(__builtin_fmaf(-c, q, a), y, q);
@@ -237,6 +268,10 @@ template <> struct Fmt<TK_E4M3> {
 template <> struct Fmt<TK_E2M1> {
     static constexpr int qmax = 6;
     static constexpr float floor_ = 6.0f * 0x1p-126f;
+};
+template <> struct Fmt<TK_E5M6> {
+    static constexpr int qmax = 65024;     // (2 - 2^-6) * 2^15
+    static constexpr float floor_ = 1e-4f;
 };
 
 // Scales of RPW rows at once.  All lanes of a group already hold the group's amax of every row, so
@@ -299,14 +334,45 @@ __device__ __forceinline__ uint32_t pack_e2m1x8(const float (&q)[8]) {
     return w;
 }
 
-// scale 8 values, convert, store: 8 bytes (E4M3) or 4 bytes (E2M1) per lane
+// fp32 -> 12-bit E5M6 code, as the reference computes it: the fp16 obtained by rounding toward zero is cut to its
+// top 12 bits, and the result is bumped by one when (kept lsb) + (low 17 bits of the fp32 pattern) exceeds 0x10000.
+// Where the fp16 is normal those 17 bits are exactly the dropped ones, i.e. round to nearest even; below 2^-14 the
+// reference uses the same bits although others were dropped, and so does this.  v_cvt_pkrtz_f16_f32 gives the
+// round-toward-zero fp16 (subnormals included) but saturates where the reference goes to infinity, hence the fix-up
+// for magnitudes from 2^16 (unreachable after scaling by 65024 / amax, kept for equality on every bit pattern).
+__device__ __forceinline__ uint32_t e5m6_code_pair(float a, float b, uint32_t &code_b) {
+    const uint32_t h2 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
+    uint32_t h[2] = {h2 & 0xFFFFu, h2 >> 16};
+    const uint32_t bits[2] = {f2u(a), f2u(b)};
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t mag = bits[i] & 0x7FFFFFFFu;
+        if (mag >= 0x47800000u) h[i] = ((bits[i] >> 16) & 0x8000u) | (mag > 0x7F800000u ? 0x7FFFu : 0x7C00u);
+        const uint32_t kept = h[i] >> 4;
+        h[i] = (kept + (((kept & 1u) + (bits[i] & 0x1FFFFu)) > 0x10000u ? 1u : 0u)) & 0xFFFu;
+    }
+    code_b = h[1];
+    return h[0];
+}
+
+__device__ __forceinline__ u32x3 pack_e5m6x8(const float (&q)[8]) {
+    uint32_t c[8];
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) c[i] = e5m6_code_pair(q[i], q[i + 1], c[i + 1]);
+    return u32x3{(c[0] << 20) | (c[1] << 8) | (c[2] >> 4),
+                 (c[2] << 28) | (c[3] << 16) | (c[4] << 4) | (c[5] >> 8),
+                 (c[5] << 24) | (c[6] << 12) | c[7]};
+}
+
+// scale 8 values, convert, store: 8 bytes (E4M3), 4 bytes (E2M1) or 12 bytes (E5M6) per lane
 template <int FMT, bool CLAMP>
 __device__ __forceinline__ void quantise_store8(const float (&v)[8], float inv, uint8_t *out_row, int col) {
     float q[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) q[i] = v[i] * inv;
     if (FMT == TK_E4M3) st_stream8(out_row + col, pack_e4m3x8<CLAMP>(q));
-    else st_stream4(out_row + (col >> 1), pack_e2m1x8(q));
+    else if (FMT == TK_E2M1) st_stream4(out_row + (col >> 1), pack_e2m1x8(q));
+    else __builtin_nontemporal_store(pack_e5m6x8(q), reinterpret_cast<u32x3 *>(out_row + (col >> 3) * 12));
 }
 
 // ---------------------------------------------------------------------------------------------

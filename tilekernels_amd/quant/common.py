@@ -14,7 +14,7 @@ from ..utils import align, ceil_div
 
 @dataclass(frozen=True)
 class CastOutputConfig:
-    fmt: str                                  # 'e4m3' | 'e2m1'
+    fmt: str                                  # 'e4m3' | 'e2m1' | 'e5m6'
     sf_block: tuple                           # (rows, cols) sharing one scale
     use_tma_aligned_col_major_sf: bool = False
     round_sf: bool = False
@@ -23,7 +23,8 @@ class CastOutputConfig:
 
     @property
     def torch_dtype(self) -> torch.dtype:
-        return torch.float8_e4m3fn if self.fmt == 'e4m3' else torch.int8    # int8 = two E2M1 codes
+        # int8 = two E2M1 codes; uint32 = a third of eight packed E5M6 codes (handed back as uint8)
+        return {'e4m3': torch.float8_e4m3fn, 'e2m1': torch.int8, 'e5m6': torch.uint32}[self.fmt]
 
     @property
     def sf_torch_dtype(self) -> torch.dtype:
@@ -31,7 +32,7 @@ class CastOutputConfig:
 
     @property
     def fmt_code(self) -> int:
-        return _ffi.TK_E4M3 if self.fmt == 'e4m3' else _ffi.TK_E2M1
+        return {'e4m3': _ffi.TK_E4M3, 'e2m1': _ffi.TK_E2M1, 'e5m6': _ffi.TK_E5M6}[self.fmt]
 
     @property
     def layout_code(self) -> int:
@@ -43,8 +44,6 @@ class CastOutputConfig:
 def get_cast_output_config(fmt, sf_block, use_tma_aligned_col_major_sf=False, round_sf=False,
                            use_packed_ue8m0=False, custom_clamp_min_value=None) -> CastOutputConfig:
     assert fmt in ('e5m6', 'e4m3', 'e2m1')
-    if fmt == 'e5m6':
-        raise NotImplementedError("fmt='e5m6' is outside this library (FP8 E4M3 / FP4 E2M1 only)")
     # one UE8M0 byte per block only exists as a power-of-two scale in the column-major packed layout
     assert not use_packed_ue8m0 or (use_tma_aligned_col_major_sf and round_sf), \
         'use_packed_ue8m0 needs use_tma_aligned_col_major_sf=True and round_sf=True'

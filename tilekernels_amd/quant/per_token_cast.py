@@ -1,4 +1,4 @@
-"""Per-token (1 x N) FP8 E4M3 / FP4 E2M1 cast: host side of tk_per_token_cast.
+"""Per-token (1 x N) FP8 E4M3 / FP4 E2M1 cast and the per-row E5M6 cast: host side of tk_per_token_cast.
 
 Signatures, defaults, asserts and return conventions follow
 tile_kernels/quant/per_token_cast_kernel.py:159-302.
@@ -24,13 +24,17 @@ def per_token_cast_impl(x, fmt, num_per_channels, x_block_size=None, use_tma_ali
     out_config = get_cast_output_config(fmt, (1, num_per_channels), use_tma_aligned_col_major_sf, round_sf, use_packed_ue8m0)
     assert x.dim() == 2 and (x.stride(1) == 1 or x.shape[1] <= 1)
     num_tokens, hidden = x.shape
-    assert num_per_channels in (16, 32, 64, 128) or (num_per_channels == hidden and hidden % 64 == 0)
-    if num_per_channels == hidden and hidden not in (16, 32, 64, 128):
-        assert not sf_only and sf is None
+    if fmt == 'e5m6':
+        # whole rows share one scale and only the full cast exists (tile_kernels/quant/per_token_cast_to_e5m6_kernel.py:172-196)
+        assert num_per_channels == hidden and hidden % 8 == 0 and not sf_only and sf is None
+    else:
+        assert num_per_channels in (16, 32, 64, 128) or (num_per_channels == hidden and hidden % 64 == 0)
+        if num_per_channels == hidden and hidden not in (16, 32, 64, 128):
+            assert not sf_only and sf is None
     dev = _ffi.require_gpu(x, sf)
     lib = _ffi.load()
 
-    out_cols = hidden if fmt == 'e4m3' else hidden // 2
+    out_cols = {'e4m3': hidden, 'e2m1': hidden // 2, 'e5m6': hidden // 8 * 3}[fmt]
     out = torch.empty((num_tokens, out_cols), dtype=out_config.torch_dtype, device=dev)
     if sf is not None:
         assert not sf_only
@@ -54,6 +58,8 @@ def per_token_cast_impl(x, fmt, num_per_channels, x_block_size=None, use_tma_ali
 
     if sf is not None:
         return out
+    if fmt == 'e5m6':
+        out = out.view(torch.uint8)
     out_sf = cast_epilogue(out_sf, num_tokens, hidden, out_config)
     return out_sf if sf_only else (out, out_sf)
 
@@ -115,7 +121,8 @@ def per_token_cast(
     use_packed_ue8m0: bool = False,
 ) -> QuantTensor:
     """Cast ``x[num_tokens, hidden]`` to FP8 (``'e4m3'``) or packed FP4 (``'e2m1'``) with one scale per
-    ``num_per_channels`` consecutive channels of a token.  Returns ``(out, out_sf)``."""
+    ``num_per_channels`` consecutive channels of a token, or to packed 12-bit ``'e5m6'`` (uint8
+    ``[num_tokens, hidden * 3 // 2]``) with one scale per token.  Returns ``(out, out_sf)``."""
     return per_token_cast_impl(x, fmt, num_per_channels, x_block_size, use_tma_aligned_col_major_sf, round_sf, use_packed_ue8m0)
 
 
