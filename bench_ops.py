@@ -347,7 +347,34 @@ def op_e5m6(direction):
     return build
 
 
+def op_lossless():
+    """FP4 1x32 (packed UE8M0 scales) -> FP8 128x128, a [7168, 2048] weight as in the per-block benchmark shape."""
+    import tilekernels_amd as tk
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    M, K = 7168, 2048
+    w = torch.randn((M, K), device='cuda', dtype=torch.bfloat16)
+    codes, sf = tk.quant.per_token_cast(w, 'e2m1', 32, use_tma_aligned_col_major_sf=True, round_sf=True, use_packed_ue8m0=True)
+    store = sf.T.view(torch.uint8)
+    out = torch.empty((M, K), device='cuda', dtype=torch.float8_e4m3fn)
+    out_sf = torch.empty((M // 128, K // 128), device='cuda', dtype=torch.float32)
+    stream = _ffi.current_stream(w.device)
+
+    def launch():
+        rc = lib.tk_per_block_cast_lossless(codes.data_ptr(), M, K, store.data_ptr(), store.stride(0), _ffi.TK_SF_COL_UE8M0, 1, 32,
+                                            out.data_ptr(), out_sf.data_ptr(), K // 128, _ffi.TK_SF_ROW_F32, 128, 128, stream)
+        assert rc == 0, rc
+    algo = codes.numel() + M * (K // 32) + nbytes(out, out_sf)
+
+    def cpu():
+        from oracle import torch_ref
+        xq = (codes.cpu(), sf.cpu())
+        return lambda: torch_ref.per_block_cast_lossless(xq, 'e4m3', (1, 32), (128, 128), round_sf=True)
+    return launch, algo, nbytes(codes, out) + store.numel(), cpu
+
+
 OPS = [
+    Op('per_block_cast_lossless', 'per_block_cast_lossless e2m1 1x32 (packed scales) -> e4m3 128x128, [7168,2048]', op_lossless),
     Op('per_token_cast_e5m6', "per_token_cast fmt='e5m6' (12-bit, one scale per row) round_sf, bf16 [8192,4096]", op_e5m6('cast')),
     Op('cast_back_e5m6', 'cast_back of e5m6 -> bf16, [8192,4096]', op_e5m6('back')),
     Op('per_token_cast_with_sf_only', 'per_token_cast_with_sf_only e4m3 1x128, bf16 [4096,7168]', op_cast_variant('token', 'sf_only')),

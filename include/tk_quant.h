@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define TK_QUANT_VERSION 107 /* major*10000 + minor*100 + patch */
+#define TK_QUANT_VERSION 108 /* major*10000 + minor*100 + patch */
 
 enum tk_dtype { TK_BF16 = 0, TK_F32 = 1 };
 enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1, TK_E5M6 = 2 };
@@ -207,6 +207,26 @@ int tk_per_channel_cast(const void *x, int x_dtype, const float *x_sf, int64_t n
 int tk_check_per_channel_cast(const void *x, int x_dtype, const float *x_sf, int64_t num_tokens, int64_t K,
                               const int32_t *pos_to_token, int64_t M, const void *out, const float *out_sf,
                               int num_per_tokens, int round_sf, int transpose, int swiglu, int use_clamp, float clamp);
+
+/*
+ * Lossless re-blocking of FP4 into FP8: x holds packed E2M1 bytes [M, K/2] (contiguous) with one power-of-two
+ * scale per x_bm x x_bk block in x_sf (any layout; of an fp32 scale only the exponent is used); out receives
+ * E4M3 bytes [M, K] with one power-of-two scale per out_bm x out_bk block:
+ *   e_out = max(exponent of x_sf over the input blocks inside the output block) - 6, not below 0
+ *   out   = code * 2^(e_in - e_out)   (exact while the input exponents of an output block span at most 11)
+ *   out_sf = 2^(e_out - 127) as fp32, or the byte e_out in the packed layout
+ * so that out * out_sf == x * x_sf for every element.
+ * Stands behind tile_kernels.quant.per_block_cast_lossless
+ * (tile_kernels/quant/per_block_cast_lossless_kernel.py:150-209).
+ *   requirements K % 8 == 0; x_bk % 8 == 0; out_bm and out_bk divide 128 and are multiples of x_bm and x_bk;
+ *                x 4-byte, out 8-byte aligned
+ */
+int tk_per_block_cast_lossless(const void *x, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld, int x_sf_layout,
+                               int x_bm, int x_bk, void *out, void *out_sf, int64_t out_sf_ld, int out_sf_layout,
+                               int out_bm, int out_bk, void *stream);
+int tk_check_per_block_cast_lossless(const void *x, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld,
+                                     int x_sf_layout, int x_bm, int x_bk, const void *out, const void *out_sf,
+                                     int64_t out_sf_ld, int out_sf_layout, int out_bm, int out_bk);
 
 /*
  * Dequantisation: out[m, k] = float(code[m, k]) * sf[m / bm, k / bk] (one fp32 product), stored as

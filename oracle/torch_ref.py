@@ -10,6 +10,8 @@ pure-torch implementations:
 * ``unpack_from_e2m1fn_x2``     <- tile_kernels/quant/common.py:247-295
 * ``encode_e2m1``               <- tile_kernels/torch/cast.py:224-252 (same result, closed form)
 * ``cast_to_e5m6`` / ``cast_back_from_e5m6`` <- tile_kernels/torch/cast_e5m6.py:145-258
+* ``per_block_cast_lossless``   <- tile_kernels/quant/per_block_cast_lossless_kernel.py:20-147 (the reference has no
+  torch statement of it; its test states the property, tests/quant/test_per_block_cast_lossless.py:90-104)
 
 Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import
 it.  The shipped package never does: it has no CPU path at all.
@@ -42,6 +44,9 @@ How each function is pinned (all pins live in tests/test_oracle_*.py and run wit
   nearest (it rounds on bits of the fp32 pattern that are not the ones dropped; cast_e5m6.py:75-81,
   per_token_cast_to_e5m6_kernel.py:49-56): that range is restated from those lines and covered only by
   hand-computed cases, so parity with the reference is unpinned there beyond those cases.
+* ``per_block_cast_lossless``: the property the reference tests (dequantising the result equals dequantising
+  the input, exactly, on its own kind of data), the closed form of the output exponent (block maximum minus 6, not
+  below 0) on hand-built inputs, and the exactness bound (a span of 11 binades) at and beyond its edge.
 """
 from typing import Optional, Tuple, Union
 
@@ -657,3 +662,25 @@ def cast_back_from_e5m6(x: QuantTensor, fmt: str, block_size: Tuple[int, int]) -
     scales = _sf_as_fp32(sf)[:_ceil_div(h, bh), :_ceil_div(w, bw)]
     out = decode_e5m6(unpack_e5m6(packed)) * _expand_blocks(scales, bh, bw, h, w)
     return out.to(torch.float32 if fmt == 'fp32' else torch.bfloat16)
+
+
+def per_block_cast_lossless(x: QuantTensor, fmt: str, x_block_size: Tuple[int, int], out_block_size: Tuple[int, int],
+                            use_tma_aligned_col_major_sf: bool = False, round_sf: bool = False,
+                            use_packed_ue8m0: bool = False) -> QuantTensor:
+    """Packed E2M1 codes with power-of-two scales per ``x_block_size`` block -> E4M3 codes with power-of-two
+    scales per ``out_block_size`` block, every value unchanged: the output exponent is the largest input
+    exponent in the block minus 6 (not below 0), each value is shifted by the difference
+    (tile_kernels/quant/per_block_cast_lossless_kernel.py:104-134)."""
+    codes, sf = x
+    assert fmt == 'e4m3' and codes.dtype == torch.int8
+    vals = unpack_from_e2m1fn_x2(codes)
+    h, w = vals.shape
+    (ibm, ibk), (obm, obk) = x_block_size, out_block_size
+    assert obm % ibm == 0 and obk % ibk == 0
+    e_in = (_sf_as_fp32(sf).contiguous().view(torch.int32) >> 23)[:_ceil_div(h, ibm), :_ceil_div(w, ibk)]
+    e_elem = _expand_blocks(e_in, ibm, ibk, h, w)
+    top = _block_amax(e_elem.to(torch.float32), obm, obk).to(torch.int32)        # exponents are small non-negative integers
+    e_out = (top - 6).clamp(min=0)
+    shift = e_elem - _expand_blocks(e_out, obm, obk, h, w)
+    out = (vals * torch.exp2(shift.to(torch.float32))).to(torch.float8_e4m3fn)
+    return out, _format_sf((e_out << 23).contiguous(), use_tma_aligned_col_major_sf, use_packed_ue8m0)

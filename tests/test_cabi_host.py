@@ -196,6 +196,32 @@ def test_per_channel_cast_validation(lib):
     assert check_pc(lib, M=0, T=0, x=0, out=0, out_sf=0) == OK
 
 
+def check_ll(lib, x=P, M=256, K=512, x_sf=P, x_ld=None, x_layout=0, ibm=1, ibk=32, out=P, out_sf=P, o_ld=None, o_layout=0, obm=128, obk=128):
+    inm, ink, onm, onk = -(-M // ibm), -(-K // ibk), -(-M // obm), -(-K // obk)
+    if x_ld is None:
+        x_ld = ink if x_layout == 0 else (inm + 3) // 4 * 4 if x_layout == 1 else (4 * inm + 15) // 16 * 16
+    if o_ld is None:
+        o_ld = onk if o_layout == 0 else (onm + 3) // 4 * 4 if o_layout == 1 else (4 * onm + 15) // 16 * 16
+    return lib.tk_check_per_block_cast_lossless(x, M, K, x_sf, x_ld, x_layout, ibm, ibk, out, out_sf, o_ld, o_layout, obm, obk)
+
+
+def test_per_block_cast_lossless_validation(lib):
+    assert check_ll(lib) == OK
+    assert check_ll(lib, obm=1) == OK and check_ll(lib, obm=32, obk=32) == OK
+    assert check_ll(lib, x_layout=2, o_layout=2) == OK
+    assert check_ll(lib, x_layout=3) == LAYOUT and check_ll(lib, o_layout=-1) == LAYOUT
+    assert check_ll(lib, K=500) == SHAPE
+    assert check_ll(lib, obk=96) == GROUP                               # output blocks divide the 128 x 128 tile
+    assert check_ll(lib, obm=256) == GROUP
+    assert check_ll(lib, ibk=64, obk=32) == GROUP                       # ... and hold whole input blocks
+    assert check_ll(lib, ibm=32, obm=1) == GROUP
+    assert check_ll(lib, ibk=4) == GROUP
+    assert check_ll(lib, x=0) == NULLP and check_ll(lib, out_sf=0) == NULLP
+    assert check_ll(lib, x=P + 2) == ALIGN and check_ll(lib, out=P + 4) == ALIGN
+    assert check_ll(lib, x_ld=3) == STRIDE and check_ll(lib, o_ld=1) == STRIDE
+    assert check_ll(lib, M=0, x=0, x_sf=0, out=0, out_sf=0) == OK
+
+
 def test_moe_layout_validation(lib):
     ws = lib.tk_fused_mapping_workspace_bytes(4096, 8, 256)
     assert ws > 0

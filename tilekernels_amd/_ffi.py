@@ -33,6 +33,8 @@ SIGNATURES = {
                                               _i64, _vp, _i32, _f32, _vp]),
     'tk_cast_back': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _i32, _vp]),
     'tk_check_cast_back': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _i32]),
+    'tk_per_block_cast_lossless': (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _vp, _i64, _i32, _i32, _i32, _vp]),
+    'tk_check_per_block_cast_lossless': (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _vp, _i64, _i32, _i32, _i32]),
     'tk_fused_mapping_workspace_bytes': (_i64, [_i64, _i32, _i32]),
     'tk_get_fused_mapping': (_i32, [_vp, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     'tk_check_get_fused_mapping': (_i32, [_vp, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64]),

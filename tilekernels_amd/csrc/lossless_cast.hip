@@ -1,0 +1,155 @@
+// Lossless re-blocking of packed FP4 E2M1 codes (power-of-two scales per small block, e.g. 1 x 32) into FP8 E4M3
+// codes with power-of-two scales per larger block (1 x 128, 32 x 32, 128 x 128, ...) for gfx950.
+//
+// Nothing is rounded.  An output block takes the exponent  e_out = max(e_in over its input blocks) - 6  (not below
+// 0), and every value becomes  code * 2^(e_in - e_out): an E2M1 magnitude (0.5 .. 6, one mantissa bit) shifted by
+// at most 6 binades up stays at or below 384 <= 448, and shifted down by at most 5 stays a normal E4M3 number, so
+// E4M3 holds it exactly as long as the input exponents of one output block differ by no more than 11.  Beyond that
+// the reference asserts (tile_kernels/quant/per_block_cast_lossless_kernel.py:126); here the small values are
+// rounded by the conversion like any other.
+//
+// A workgroup of 256 threads owns a 128 x 128 tile (every supported output block divides it): a lane takes 8
+// consecutive codes (4 bytes) of rows r, r + 16, ..., 8 in all, each with the exponent of its input block.  The
+// exponent maxima of the output blocks are formed along the rows with DPP (the 16 lanes of a tile row are one DPP row),
+// down a lane's own rows in registers, and across lanes and waves with a few integer atomics on a small LDS table; then every lane shifts, converts and stores 8 bytes per
+// row, and the first threads store the tile's output scales.
+//
+// Reference semantics: tile_kernels/quant/per_block_cast_lossless_kernel.py:15-147 (kernel) and :150-209 (wrapper).
+#include "tk_device.hpp"
+#include "tk_host.hpp"
+
+namespace tk {
+
+constexpr int kLlTile = 128;                          // rows and columns per tile
+constexpr int kLlPieces = kLlTile / 8;                // 8-code pieces per tile row = lanes per row: 16
+constexpr int kLlRowsPerPass = kThreads / kLlPieces;  // 16
+constexpr int kLlPasses = kLlTile / kLlRowsPerPass;   // 8 rows per lane
+
+__global__ __launch_bounds__(kThreads) void lossless_fp4_to_fp8_kernel(const uint8_t *x, void *a_xsf, int64_t a_xsf_ld, int M, int K,
+                                                                       int a_xsf_layout, int ibm_sh, int ibk_sh, int obm_sh, int obk_sh,
+                                                                       uint8_t *out, void *a_sf, int64_t a_sf_ld, int a_sf_layout,
+                                                                       int in_nm, int in_nk, int out_nm, int out_nk) {
+    const SfRef xsf{a_xsf, a_xsf_ld, a_xsf_layout, in_nm, in_nk};
+    const SfRef sf{a_sf, a_sf_ld, a_sf_layout, out_nm, out_nk};
+    __shared__ int32_t blk_max[kLlTile][kLlPieces];   // [output block row][output block column] of the tile; at most 128 x 16 used
+    const int tile_m = blockIdx.y, tile_k = blockIdx.x;
+    const int piece = threadIdx.x % kLlPieces, r0 = threadIdx.x / kLlPieces;
+    const int col = tile_k * kLlTile + piece * 8;
+    const bool col_ok = col < K;
+    // every block extent is a power of two (the output blocks divide 128, the input blocks divide them): shifts, no divisions
+    const int bcols_sh = 7 - obk_sh, bcols = 1 << bcols_sh, brows = kLlTile >> obm_sh;   // output blocks of a tile along the columns / rows
+    const int lpb_sh = obk_sh - 3, lanes_per_block = 1 << lpb_sh;   // pieces of a row inside one output block: 1, 2, 4, 8 or 16
+    const int bk_idx = piece >> lpb_sh;
+
+    for (int i = threadIdx.x; i < brows * bcols; i += kThreads) blk_max[i >> bcols_sh][i & (bcols - 1)] = 0;
+
+    // All loads first, without a branch around them (a branch per row makes the compiler finish one row's loads
+    // before it issues the next): rows and columns outside the matrix read the tile's first element and count as 0.
+    uint32_t code[kLlPasses];
+    int e_in[kLlPasses];
+    const int row_first = tile_m * kLlTile, col_first = tile_k * kLlTile;
+#pragma unroll
+    for (int p = 0; p < kLlPasses; ++p) {
+        const int row = row_first + p * kLlRowsPerPass + r0;
+        const bool ok = col_ok && row < M;
+        const int rr = ok ? row : row_first, cc = ok ? col : col_first;
+        code[p] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(x + (((int64_t)rr * K + cc) >> 1)));
+        e_in[p] = (int)(f2u(sf_load_select(xsf, rr >> ibm_sh, cc >> ibk_sh)) >> 23);
+        if (!ok) { code[p] = 0u; e_in[p] = 0; }
+    }
+
+    __syncthreads();
+    // Block maxima.  Along a row: the 16 lanes of a tile row are one DPP row, so the lanes that share an output block
+    // reduce without LDS.  Down the rows: a lane folds its own consecutive rows while they stay in one block, and
+    // only then does the first lane of each group touch the LDS table (16 atomics per 128 x 128 block, not 2048).
+    uint32_t run = 0u;
+#pragma unroll
+    for (int p = 0; p < kLlPasses; ++p) {
+        uint32_t m = (uint32_t)e_in[p];
+        if (lanes_per_block >= 2) m = umax(m, dpp_u32<kDppXor1>(m));
+        if (lanes_per_block >= 4) m = umax(m, dpp_u32<kDppXor2>(m));
+        if (lanes_per_block >= 8) m = umax(m, dpp_u32<kDppHalfMirror>(m));
+        if (lanes_per_block >= 16) m = umax(m, dpp_u32<kDppMirror>(m));
+        run = umax(run, m);
+        const int br = (p * kLlRowsPerPass + r0) >> obm_sh;
+        const int br_next = p + 1 < kLlPasses ? ((p + 1) * kLlRowsPerPass + r0) >> obm_sh : -1;
+        if (br != br_next) {
+            if ((piece & (lanes_per_block - 1)) == 0 && run != 0u) atomicMax(&blk_max[br][bk_idx], (int32_t)run);
+            run = 0u;
+        }
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int p = 0; p < kLlPasses; ++p) {
+        const int row_in_tile = p * kLlRowsPerPass + r0;
+        const int row = tile_m * kLlTile + row_in_tile;
+        if (!(col_ok && row < M)) continue;
+        const int top = blk_max[row_in_tile >> obm_sh][bk_idx];
+        const int e_out = top >= 6 ? top - 6 : 0;
+        // 2^(e_in - e_out) as a float: biased exponent e_in - e_out + 127, which the reference lets wrap when the input
+        // exponents of a block are further apart than it supports
+        Raw8<e2m1in_t> raw;
+        raw.w = code[p];
+        raw.s = u2f((uint32_t)(e_in[p] - e_out + 127) << 23);
+        float v[8];
+        raw.get(v);
+        st_stream8(out + (int64_t)row * K + col, pack_e4m3x8<false>(v));
+    }
+
+    for (int i = threadIdx.x; i < brows * bcols; i += kThreads) {
+        const int bm_i = i >> bcols_sh, bk_i = i & (bcols - 1);
+        const int m = tile_m * brows + bm_i, k = tile_k * bcols + bk_i;
+        if (m < out_nm && k < out_nk) {
+            const int top = blk_max[bm_i][bk_i];
+            Scale sc;
+            sc.e8 = (uint32_t)(top >= 6 ? top - 6 : 0);
+            sc.sf = u2f(sc.e8 << 23);
+            sc.inv = 0.0f;
+            sf_store(sf, m, k, sc);
+        }
+    }
+}
+
+}  // namespace tk
+
+using namespace tk;
+
+extern "C" int tk_check_per_block_cast_lossless(const void *x, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld,
+                                                int x_sf_layout, int x_bm, int x_bk, const void *out, const void *out_sf,
+                                                int64_t out_sf_ld, int out_sf_layout, int out_bm, int out_bk) {
+    if (x_sf_layout < TK_SF_ROW_F32 || x_sf_layout > TK_SF_COL_UE8M0) return TK_ERR_BAD_LAYOUT;
+    if (out_sf_layout < TK_SF_ROW_F32 || out_sf_layout > TK_SF_COL_UE8M0) return TK_ERR_BAD_LAYOUT;
+    if (M < 0 || K <= 0 || K % 8 != 0) return TK_ERR_BAD_SHAPE;
+    if (M > INT32_MAX - 256 || K > INT32_MAX - 256) return TK_ERR_TOO_LARGE;
+    if (x_bm < 1 || x_bk < 8 || x_bk % 8 != 0) return TK_ERR_BAD_GROUP;
+    // output blocks divide the 128 x 128 tile, hold whole 8-code pieces and whole input blocks
+    if (out_bm < 1 || out_bk < 8 || kLlTile % out_bm != 0 || kLlTile % out_bk != 0 || out_bk % 8 != 0) return TK_ERR_BAD_GROUP;
+    if (out_bm % x_bm != 0 || out_bk % x_bk != 0) return TK_ERR_BAD_GROUP;
+    if (M == 0) return TK_OK;
+    if (!x || !x_sf || !out || !out_sf) return TK_ERR_NULL_POINTER;
+    if (!aligned_to(x, 4) || !aligned_to(out, 8) || !aligned_to(x_sf, 4) || !aligned_to(out_sf, 4)) return TK_ERR_MISALIGNED;
+    const int64_t inm = (M + x_bm - 1) / x_bm, ink = (K + x_bk - 1) / x_bk;
+    const int64_t onm = (M + out_bm - 1) / out_bm, onk = (K + out_bk - 1) / out_bk;
+    const int64_t xneed = x_sf_layout == TK_SF_ROW_F32 ? ink : (x_sf_layout == TK_SF_COL_F32 ? inm : 4 * inm);
+    const int64_t oneed = out_sf_layout == TK_SF_ROW_F32 ? onk : (out_sf_layout == TK_SF_COL_F32 ? onm : 4 * onm);
+    if (x_sf_ld < xneed || out_sf_ld < oneed) return TK_ERR_BAD_STRIDE;
+    if (out_sf_layout == TK_SF_COL_UE8M0 && out_sf_ld % 4 != 0) return TK_ERR_MISALIGNED;
+    if ((M + kLlTile - 1) / kLlTile > 65535) return TK_ERR_TOO_LARGE;   // row tiles ride on grid.y
+    return TK_OK;
+}
+
+extern "C" int tk_per_block_cast_lossless(const void *x, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld, int x_sf_layout,
+                                          int x_bm, int x_bk, void *out, void *out_sf, int64_t out_sf_ld, int out_sf_layout,
+                                          int out_bm, int out_bk, void *stream) {
+    const int rc = tk_check_per_block_cast_lossless(x, M, K, x_sf, x_sf_ld, x_sf_layout, x_bm, x_bk, out, out_sf, out_sf_ld,
+                                                    out_sf_layout, out_bm, out_bk);
+    if (rc != TK_OK || M == 0) return rc;
+    const dim3 grid((unsigned)((K + kLlTile - 1) / kLlTile), (unsigned)((M + kLlTile - 1) / kLlTile));
+    auto log2i = [](int v) { int s = 0; while ((1 << s) < v) ++s; return s; };
+    hipLaunchKernelGGL(lossless_fp4_to_fp8_kernel, grid, dim3(kThreads), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint8_t *>(x), const_cast<void *>(x_sf), x_sf_ld, (int)M, (int)K, x_sf_layout, log2i(x_bm), log2i(x_bk),
+                       log2i(out_bm), log2i(out_bk), static_cast<uint8_t *>(out), out_sf, out_sf_ld, out_sf_layout, (int)((M + x_bm - 1) / x_bm),
+                       (int)((K + x_bk - 1) / x_bk), (int)((M + out_bm - 1) / out_bm), (int)((K + out_bk - 1) / out_bk));
+    return (int)hipGetLastError();
+}
