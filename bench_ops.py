@@ -373,7 +373,39 @@ def op_lossless():
     return launch, algo, nbytes(codes, out) + store.numel(), cpu
 
 
+def op_reduce_fused(fp8):
+    """The inverse of expand_to_fused at its benchmark shape: bf16 [R, 4096] expanded rows -> [4096, 4096] tokens, top-8."""
+    def build():
+        from tilekernels_amd import _ffi
+        lib = _ffi.load()
+        T, K, hidden = 4096, 8, 4096
+        _, maps = _moe_maps(T, K)
+        p2e, t2p = maps[0], maps[3]
+        R = p2e.numel()
+        x = torch.randn((R, hidden), device='cuda', dtype=torch.bfloat16)
+        w = torch.rand((T, K), device='cuda')
+        sf = torch.ones((1,), device='cuda')
+        out = torch.empty((T, hidden), device='cuda', dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16)
+        stream = _ffi.current_stream(x.device)
+
+        def launch():
+            rc = lib.tk_reduce_fused(x.data_ptr(), _ffi.TK_BF16, R, hidden, 0, w.data_ptr(), t2p.data_ptr(), T, K, out.data_ptr(),
+                                     _ffi.TK_OUT_E4M3 if fp8 else _ffi.TK_BF16, sf.data_ptr() if fp8 else 0, stream)
+            assert rc == 0, rc
+        # the T * K live rows are read, padding rows are not
+        algo = T * K * hidden * 2 + nbytes(out, w, t2p)
+
+        def cpu():
+            from oracle import torch_ref
+            xc, wc, tc, sc = x.cpu(), w.cpu(), t2p.cpu(), sf.cpu()
+            return lambda: torch_ref.reduce_fused(xc, wc, tc, 'e4m3' if fp8 else '', sc if fp8 else None)
+        return launch, algo, nbytes(x, out), cpu
+    return build
+
+
 OPS = [
+    Op('reduce_fused', 'reduce_fused bf16 [R,4096] -> bf16 [4096,4096], top-8 of 256 experts, weighted', op_reduce_fused(False)),
+    Op('reduce_fused_fp8', 'reduce_fused bf16 [R,4096] -> e4m3 [4096,4096] with output scale, top-8, weighted', op_reduce_fused(True)),
     Op('per_block_cast_lossless', 'per_block_cast_lossless e2m1 1x32 (packed scales) -> e4m3 128x128, [7168,2048]', op_lossless),
     Op('per_token_cast_e5m6', "per_token_cast fmt='e5m6' (12-bit, one scale per row) round_sf, bf16 [8192,4096]", op_e5m6('cast')),
     Op('cast_back_e5m6', 'cast_back of e5m6 -> bf16, [8192,4096]', op_e5m6('back')),

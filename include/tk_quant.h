@@ -37,9 +37,9 @@
 extern "C" {
 #endif
 
-#define TK_QUANT_VERSION 108 /* major*10000 + minor*100 + patch */
+#define TK_QUANT_VERSION 109 /* major*10000 + minor*100 + patch */
 
-enum tk_dtype { TK_BF16 = 0, TK_F32 = 1 };
+enum tk_dtype { TK_BF16 = 0, TK_F32 = 1, TK_OUT_E4M3 = 2 /* output of tk_reduce_fused only */ };
 enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1, TK_E5M6 = 2 };
 enum tk_sf_layout { TK_SF_ROW_F32 = 0, TK_SF_COL_F32 = 1, TK_SF_COL_UE8M0 = 2 };
 enum tk_mode {
@@ -207,6 +207,23 @@ int tk_per_channel_cast(const void *x, int x_dtype, const float *x_sf, int64_t n
 int tk_check_per_channel_cast(const void *x, int x_dtype, const float *x_sf, int64_t num_tokens, int64_t K,
                               const int32_t *pos_to_token, int64_t M, const void *out, const float *out_sf,
                               int num_per_tokens, int round_sf, int transpose, int swiglu, int use_clamp, float clamp);
+
+/*
+ * Weighted reduction of expanded rows back to tokens (the inverse of tk_expand_to_fused):
+ *   out[t, :] = round( sf * sum_k  x[pos, :] * (topk_weights[t, k] * x_sf[pos]) ),   pos = token_topk_to_pos[t, k] >= 0
+ * accumulated in fp32 with one fused multiply-add per term, k ascending; topk_weights, x_sf ([num_expanded]
+ * fp32) and sf (one fp32 on the device) may each be NULL (factor 1).  x: bf16 or fp32 [num_expanded, hidden],
+ * contiguous; out: the type of x, or E4M3 bytes with out_dtype = TK_OUT_E4M3.
+ * Stands behind tile_kernels.moe.reduce_fused (tile_kernels/moe/reduce_fused_kernel.py:70-135; oracle
+ * tile_kernels/torch/reduce_fused.py:14-72).
+ *   requirements hidden % 8 == 0; x and out 16-byte (E4M3 out: 8-byte) aligned
+ */
+int tk_reduce_fused(const void *x, int x_dtype, int64_t num_expanded, int64_t hidden, const float *x_sf,
+                    const float *topk_weights, const int32_t *token_topk_to_pos, int64_t num_tokens, int num_topk, void *out,
+                    int out_dtype, const float *sf, void *stream);
+int tk_check_reduce_fused(const void *x, int x_dtype, int64_t num_expanded, int64_t hidden, const float *x_sf,
+                          const float *topk_weights, const int32_t *token_topk_to_pos, int64_t num_tokens, int num_topk,
+                          const void *out, int out_dtype, const float *sf);
 
 /*
  * Lossless re-blocking of FP4 into FP8: x holds packed E2M1 bytes [M, K/2] (contiguous) with one power-of-two

@@ -10,6 +10,7 @@ pure-torch implementations:
 * ``unpack_from_e2m1fn_x2``     <- tile_kernels/quant/common.py:247-295
 * ``encode_e2m1``               <- tile_kernels/torch/cast.py:224-252 (same result, closed form)
 * ``cast_to_e5m6`` / ``cast_back_from_e5m6`` <- tile_kernels/torch/cast_e5m6.py:145-258
+* ``reduce_fused``              <- tile_kernels/torch/reduce_fused.py:14-72
 * ``per_block_cast_lossless``   <- tile_kernels/quant/per_block_cast_lossless_kernel.py:20-147 (the reference has no
   torch statement of it; its test states the property, tests/quant/test_per_block_cast_lossless.py:90-104)
 
@@ -47,6 +48,9 @@ How each function is pinned (all pins live in tests/test_oracle_*.py and run wit
 * ``per_block_cast_lossless``: the property the reference tests (dequantising the result equals dequantising
   the input, exactly, on its own kind of data), the closed form of the output exponent (block maximum minus 6, not
   below 0) on hand-built inputs, and the exactness bound (a span of 11 binades) at and beyond its edge.
+* ``reduce_fused``: a float64 evaluation (bounds the whole sum), a naive Python loop over tokens and terms built on
+  the C library's ``fmaf`` (fixes the order of accumulation and the single rounding per term), hand cases for
+  skipped positions, missing weights, row factors, the final scale and each output type.
 """
 from typing import Optional, Tuple, Union
 
@@ -684,3 +688,31 @@ def per_block_cast_lossless(x: QuantTensor, fmt: str, x_block_size: Tuple[int, i
     shift = e_elem - _expand_blocks(e_out, obm, obk, h, w)
     out = (vals * torch.exp2(shift.to(torch.float32))).to(torch.float8_e4m3fn)
     return out, _format_sf((e_out << 23).contiguous(), use_tma_aligned_col_major_sf, use_packed_ue8m0)
+
+
+def reduce_fused(x: Union[torch.Tensor, QuantTensor], topk_weights: Optional[torch.Tensor], token_topk_to_pos: torch.Tensor,
+                 fp8_format: str = '', sf: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[t] = sum_k x[pos[t, k]] * (w[t, k] * x_sf[pos[t, k]])`` over the positions >= 0, accumulated in fp32 with one
+    fused multiply-add per term in the order of k, times ``sf[0]``, rounded to the dtype of ``x`` or to E4M3
+    (tile_kernels/torch/reduce_fused.py:14-72)."""
+    x_sf = None
+    if isinstance(x, tuple):
+        x, x_sf = x
+    hidden = x.shape[1]
+    num_tokens, num_topk = token_topk_to_pos.shape
+    out_dtype = torch.float8_e4m3fn if fp8_format == 'e4m3' else x.dtype
+    if num_tokens == 0:
+        return torch.empty((0, hidden), dtype=out_dtype)
+    acc = torch.zeros((num_tokens, hidden), dtype=torch.float32)
+    for k in range(num_topk):
+        pos = token_topk_to_pos[:, k].long()
+        live = pos >= 0
+        src = pos.clamp(min=0)
+        s = topk_weights[:, k].clone() if topk_weights is not None else torch.ones(num_tokens, dtype=torch.float32)
+        if x_sf is not None:
+            s = s * x_sf[src]
+        term = fma_f32(x[src].to(torch.float32), s.unsqueeze(1), acc)
+        acc = torch.where(live.unsqueeze(1), term, acc)
+    if sf is not None:
+        acc = acc * sf[0]
+    return acc.to(out_dtype)

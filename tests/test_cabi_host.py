@@ -222,6 +222,22 @@ def test_per_block_cast_lossless_validation(lib):
     assert check_ll(lib, M=0, x=0, x_sf=0, out=0, out_sf=0) == OK
 
 
+def check_rf(lib, x=P, dt=0, R=1024, hidden=2048, x_sf=0, w=0, pos=P, T=128, K=8, out=P, odt=None, sf=0):
+    return lib.tk_check_reduce_fused(x, dt, R, hidden, x_sf, w, pos, T, K, out, dt if odt is None else odt, sf)
+
+
+def test_reduce_fused_validation(lib):
+    assert check_rf(lib) == OK and check_rf(lib, dt=1) == OK
+    assert check_rf(lib, odt=2) == OK and check_rf(lib, dt=1, odt=2, sf=P, w=P, x_sf=P) == OK     # FP8 output
+    assert check_rf(lib, dt=0, odt=1) == DTYPE                          # otherwise the output has the input's type
+    assert check_rf(lib, dt=2) == DTYPE
+    assert check_rf(lib, hidden=2052) == SHAPE and check_rf(lib, K=0) == SHAPE
+    assert check_rf(lib, pos=0) == NULLP and check_rf(lib, out=0) == NULLP and check_rf(lib, x=0) == NULLP
+    assert check_rf(lib, x=P + 8) == ALIGN and check_rf(lib, out=P + 8) == ALIGN
+    assert check_rf(lib, out=P + 8, odt=2) == OK                        # FP8 rows need 8-byte alignment only
+    assert check_rf(lib, T=0, pos=0, out=0, x=0) == OK
+
+
 def test_moe_layout_validation(lib):
     ws = lib.tk_fused_mapping_workspace_bytes(4096, 8, 256)
     assert ws > 0

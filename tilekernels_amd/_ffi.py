@@ -10,7 +10,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library links against bef
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, 'lib', 'libtk_quant.so')
 
-TK_BF16, TK_F32 = 0, 1
+TK_BF16, TK_F32, TK_OUT_E4M3 = 0, 1, 2
 TK_E4M3, TK_E2M1, TK_E5M6 = 0, 1, 2
 TK_SF_ROW_F32, TK_SF_COL_F32, TK_SF_COL_UE8M0 = 0, 1, 2
 TK_CAST_AND_SF, TK_SF_ONLY, TK_CAST_GIVEN_SF = 0, 1, 2
@@ -35,6 +35,8 @@ SIGNATURES = {
     'tk_check_cast_back': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _i32]),
     'tk_per_block_cast_lossless': (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _vp, _i64, _i32, _i32, _i32, _vp]),
     'tk_check_per_block_cast_lossless': (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _vp, _i64, _i32, _i32, _i32]),
+    'tk_reduce_fused': (_i32, [_vp, _i32, _i64, _i64, _vp, _vp, _vp, _i64, _i32, _vp, _i32, _vp, _vp]),
+    'tk_check_reduce_fused': (_i32, [_vp, _i32, _i64, _i64, _vp, _vp, _vp, _i64, _i32, _vp, _i32, _vp]),
     'tk_fused_mapping_workspace_bytes': (_i64, [_i64, _i32, _i32]),
     'tk_get_fused_mapping': (_i32, [_vp, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     'tk_check_get_fused_mapping': (_i32, [_vp, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64]),

@@ -3,7 +3,8 @@
 // work, HBM- and latency-bound; no LDS tiling beyond per-wave histograms.
 //
 // Reference semantics: tile_kernels/moe/get_fused_mapping_kernel.py:24-250,
-// tile_kernels/moe/expand_to_fused_kernel.py:16-200, tile_kernels/torch/expand_to_fused.py.
+// tile_kernels/moe/expand_to_fused_kernel.py:16-200, tile_kernels/torch/expand_to_fused.py,
+// tile_kernels/moe/reduce_fused_kernel.py:12-135, tile_kernels/torch/reduce_fused.py.
 #include "tk_device.hpp"
 #include "tk_host.hpp"
 
@@ -229,6 +230,78 @@ __global__ __launch_bounds__(kThreads) void expand_to_fused_kernel(const uint8_t
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// reduce_fused: the inverse of the expansion.  out[t] = sum over k of x[pos(t, k)] * s(t, k), accumulated in fp32 with
+// one fused multiply-add per term, in the order k = 0, 1, ... (so that results are reproducible bit for bit), where
+// s = topk_weights[t, k] (or 1) times x_sf[pos] (if given); positions < 0 are skipped.  The sum is scaled by *sf (if
+// given) and rounded to the output type.  A thread owns 8 consecutive elements of one token: up to 8 rows' pieces are
+// loaded before the first is used, and there is one store per thread.
+constexpr int kReduceUnroll = 8;
+
+template <typename InT> struct ReduceIn;
+template <> struct ReduceIn<bf16_t> { typedef Raw8<bf16_t> raw; };
+template <> struct ReduceIn<float> { typedef Raw8<float> raw; };
+
+// OUT: 0 bf16, 1 fp32, 2 E4M3
+template <typename InT, int OUT>
+__global__ __launch_bounds__(kThreads) void reduce_fused_kernel(const InT *x, const int32_t *token_topk_to_pos, int num_topk, int hidden,
+                                                                int num_expanded, const float *topk_weights, const float *x_sf,
+                                                                const float *sf, void *out) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const int t = blockIdx.y;
+    const int col = (blockIdx.x * kThreads + threadIdx.x) * 8;
+    if (col >= hidden) return;
+    const int32_t *pos_row = token_topk_to_pos + (int64_t)t * num_topk;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    for (int k0 = 0; k0 < num_topk; k0 += kReduceUnroll) {
+        typename ReduceIn<InT>::raw raw[kReduceUnroll];
+        float s[kReduceUnroll];
+        bool live[kReduceUnroll];
+#pragma unroll
+        for (int j = 0; j < kReduceUnroll; ++j) {
+            const int k = k0 + j;
+            const int p = k < num_topk ? uniform_load(pos_row + k) : -1;
+            live[j] = p >= 0 && p < num_expanded;
+            // a skipped term reads row 0 (no branch around the loads) and is not added
+            const int row = live[j] ? p : 0;
+            raw[j].load(x + (int64_t)row * hidden + col);
+            s[j] = 1.0f;
+            if (topk_weights) s[j] = live[j] ? uniform_load(topk_weights + (int64_t)t * num_topk + k) : 0.0f;
+            if (x_sf) s[j] = s[j] * uniform_load(x_sf + row);
+        }
+#pragma unroll
+        for (int j = 0; j < kReduceUnroll; ++j) {
+            if (!live[j]) continue;      // wave-uniform
+            float v[8];
+            raw[j].get(v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(v[i], s[j], acc[i]);
+        }
+    }
+    if (sf) {
+        const float f = uniform_load(sf);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = acc[i] * f;
+    }
+    const int64_t idx = (int64_t)t * hidden + col;
+    if (OUT == 1) {
+        u32x4 *o = reinterpret_cast<u32x4 *>(reinterpret_cast<float *>(out) + idx);
+        __builtin_nontemporal_store(u32x4{f2u(acc[0]), f2u(acc[1]), f2u(acc[2]), f2u(acc[3])}, o);
+        __builtin_nontemporal_store(u32x4{f2u(acc[4]), f2u(acc[5]), f2u(acc[6]), f2u(acc[7])}, o + 1);
+    } else if (OUT == 0) {
+        u32x4 w;
+        w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{acc[0], acc[1]}), bf16x2));
+        w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{acc[2], acc[3]}), bf16x2));
+        w.z = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{acc[4], acc[5]}), bf16x2));
+        w.w = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{acc[6], acc[7]}), bf16x2));
+        __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(out) + idx));
+    } else {
+        st_stream8(reinterpret_cast<uint8_t *>(out) + idx, pack_e4m3x8<false>(acc));
+    }
+}
+
 }  // namespace tk
 
 using namespace tk;
@@ -331,5 +404,54 @@ extern "C" int tk_expand_to_fused(const void *x, int64_t num_tokens, int64_t row
                        static_cast<const uint8_t *>(x), row_bytes, token_topk_to_pos, num_topk, (int)chunks, (int)copy_blocks,
                        (int)num_tokens, (int)num_expanded, static_cast<uint8_t *>(out), pos_to_expert,
                        static_cast<const uint32_t *>(x_sf), sf_cols, static_cast<uint32_t *>(out_sf), out_sf_ld, sf_col_major, pad_rows);
+    return (int)hipGetLastError();
+}
+
+extern "C" int tk_check_reduce_fused(const void *x, int x_dtype, int64_t num_expanded, int64_t hidden, const float *x_sf,
+                                     const float *topk_weights, const int32_t *token_topk_to_pos, int64_t num_tokens, int num_topk,
+                                     const void *out, int out_dtype, const float *sf) {
+    (void)x_sf;
+    (void)topk_weights;
+    (void)sf;
+    if (x_dtype != TK_BF16 && x_dtype != TK_F32) return TK_ERR_BAD_DTYPE;
+    if (out_dtype != x_dtype && out_dtype != TK_OUT_E4M3) return TK_ERR_BAD_DTYPE;      // same type as the input, or FP8
+    if (num_tokens < 0 || num_expanded < 0 || num_topk <= 0 || hidden <= 0 || hidden % 8 != 0) return TK_ERR_BAD_SHAPE;
+    if (num_tokens > 65535LL * 65535 || num_expanded > INT32_MAX - 1 || hidden > INT32_MAX - 4096) return TK_ERR_TOO_LARGE;
+    if (num_tokens == 0) return TK_OK;
+    if (!token_topk_to_pos || !out) return TK_ERR_NULL_POINTER;
+    if (num_expanded > 0 && !x) return TK_ERR_NULL_POINTER;
+    if (!aligned_to(x, 16) || !aligned_to(out, out_dtype == TK_OUT_E4M3 ? 8 : 16)) return TK_ERR_MISALIGNED;
+    if (x_dtype == TK_F32 && !aligned_to(x, 16)) return TK_ERR_MISALIGNED;
+    return TK_OK;
+}
+
+extern "C" int tk_reduce_fused(const void *x, int x_dtype, int64_t num_expanded, int64_t hidden, const float *x_sf,
+                               const float *topk_weights, const int32_t *token_topk_to_pos, int64_t num_tokens, int num_topk,
+                               void *out, int out_dtype, const float *sf, void *stream) {
+    const int rc = tk_check_reduce_fused(x, x_dtype, num_expanded, hidden, x_sf, topk_weights, token_topk_to_pos, num_tokens,
+                                         num_topk, out, out_dtype, sf);
+    if (rc != TK_OK || num_tokens == 0) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned chunks = (unsigned)((hidden + kThreads * 8 - 1) / (kThreads * 8));
+    // tokens ride on grid.y (at most 65535 per launch)
+    for (int64_t t0 = 0; t0 < num_tokens; t0 += 65535) {
+        const unsigned nt = (unsigned)(num_tokens - t0 < 65535 ? num_tokens - t0 : 65535);
+        const dim3 grid(chunks, nt);
+        const int32_t *pos = token_topk_to_pos + t0 * num_topk;
+        const float *w = topk_weights ? topk_weights + t0 * num_topk : nullptr;
+        const int64_t out_bytes = out_dtype == TK_F32 ? 4 : (out_dtype == TK_BF16 ? 2 : 1);
+        void *o = static_cast<uint8_t *>(out) + t0 * hidden * out_bytes;
+#define TK_REDUCE_LAUNCH(T, O)                                                                                              \
+    hipLaunchKernelGGL((reduce_fused_kernel<T, O>), grid, dim3(kThreads), 0, s, static_cast<const T *>(x), pos, num_topk, (int)hidden, \
+                       (int)num_expanded, w, x_sf, sf, o)
+        if (x_dtype == TK_BF16) {
+            if (out_dtype == TK_OUT_E4M3) TK_REDUCE_LAUNCH(bf16_t, 2);
+            else TK_REDUCE_LAUNCH(bf16_t, 0);
+        } else {
+            if (out_dtype == TK_OUT_E4M3) TK_REDUCE_LAUNCH(float, 2);
+            else TK_REDUCE_LAUNCH(float, 1);
+        }
+#undef TK_REDUCE_LAUNCH
+    }
     return (int)hipGetLastError();
 }
