@@ -8,9 +8,9 @@
 // the reference asserts (tile_kernels/quant/per_block_cast_lossless_kernel.py:126); here the small values are
 // rounded by the conversion like any other.
 //
-// A workgroup of 256 threads owns a 128 x 128 tile (every supported output block divides it): a lane takes 8
+// A workgroup of 512 threads owns a 128 x 256 tile (every supported output block divides 128 x 128): a lane takes 8
 // consecutive codes (4 bytes) of rows r, r + 16, ..., 8 in all, each with the exponent of its input block.  The
-// exponent maxima of the output blocks are formed along the rows with DPP (the 16 lanes of a tile row are one DPP row),
+// exponent maxima of the output blocks are formed along the rows with DPP (a tile row is two DPP rows of 16 lanes, 128 columns each),
 // down a lane's own rows in registers, and across lanes and waves with a few integer atomics on a small LDS table; then every lane shifts, converts and stores 8 bytes per
 // row, and the first threads store the tile's output scales.
 //
@@ -20,34 +20,37 @@
 
 namespace tk {
 
-constexpr int kLlTile = 128;                          // rows and columns per tile
-constexpr int kLlPieces = kLlTile / 8;                // 8-code pieces per tile row = lanes per row: 16
-constexpr int kLlRowsPerPass = kThreads / kLlPieces;  // 16
-constexpr int kLlPasses = kLlTile / kLlRowsPerPass;   // 8 rows per lane
+constexpr int kLlTile = 128;                            // rows per tile; also the largest output block extent
+constexpr int kLlTileK = 256;                           // columns per tile: a tile row is 128 bytes of codes, one whole cache line
+                                                        // (with 128 columns, two workgroups fetched each line: 2.0 x the reads)
+constexpr int kLlThreads = 512;
+constexpr int kLlPieces = kLlTileK / 8;                 // 8-code pieces per tile row = lanes per row: 32 (two DPP rows)
+constexpr int kLlRowsPerPass = kLlThreads / kLlPieces;  // 16
+constexpr int kLlPasses = kLlTile / kLlRowsPerPass;     // 8 rows per lane
 
-__global__ __launch_bounds__(kThreads) void lossless_fp4_to_fp8_kernel(const uint8_t *x, void *a_xsf, int64_t a_xsf_ld, int M, int K,
+__global__ __launch_bounds__(kLlThreads) void lossless_fp4_to_fp8_kernel(const uint8_t *x, void *a_xsf, int64_t a_xsf_ld, int M, int K,
                                                                        int a_xsf_layout, int ibm_sh, int ibk_sh, int obm_sh, int obk_sh,
                                                                        uint8_t *out, void *a_sf, int64_t a_sf_ld, int a_sf_layout,
                                                                        int in_nm, int in_nk, int out_nm, int out_nk) {
     const SfRef xsf{a_xsf, a_xsf_ld, a_xsf_layout, in_nm, in_nk};
     const SfRef sf{a_sf, a_sf_ld, a_sf_layout, out_nm, out_nk};
-    __shared__ int32_t blk_max[kLlTile][kLlPieces];   // [output block row][output block column] of the tile; at most 128 x 16 used
+    __shared__ int32_t blk_max[kLlTile][kLlPieces];   // [output block row][output block column] of the tile; at most 128 x 32 used
     const int tile_m = blockIdx.y, tile_k = blockIdx.x;
     const int piece = threadIdx.x % kLlPieces, r0 = threadIdx.x / kLlPieces;
-    const int col = tile_k * kLlTile + piece * 8;
+    const int col = tile_k * kLlTileK + piece * 8;
     const bool col_ok = col < K;
     // every block extent is a power of two (the output blocks divide 128, the input blocks divide them): shifts, no divisions
-    const int bcols_sh = 7 - obk_sh, bcols = 1 << bcols_sh, brows = kLlTile >> obm_sh;   // output blocks of a tile along the columns / rows
+    const int bcols_sh = 8 - obk_sh, bcols = 1 << bcols_sh, brows = kLlTile >> obm_sh;   // output blocks of a tile along the columns / rows
     const int lpb_sh = obk_sh - 3, lanes_per_block = 1 << lpb_sh;   // pieces of a row inside one output block: 1, 2, 4, 8 or 16
     const int bk_idx = piece >> lpb_sh;
 
-    for (int i = threadIdx.x; i < brows * bcols; i += kThreads) blk_max[i >> bcols_sh][i & (bcols - 1)] = 0;
+    for (int i = threadIdx.x; i < brows * bcols; i += kLlThreads) blk_max[i >> bcols_sh][i & (bcols - 1)] = 0;
 
     // All loads first, without a branch around them (a branch per row makes the compiler finish one row's loads
     // before it issues the next): rows and columns outside the matrix read the tile's first element and count as 0.
     uint32_t code[kLlPasses];
     int e_in[kLlPasses];
-    const int row_first = tile_m * kLlTile, col_first = tile_k * kLlTile;
+    const int row_first = tile_m * kLlTile, col_first = tile_k * kLlTileK;
 #pragma unroll
     for (int p = 0; p < kLlPasses; ++p) {
         const int row = row_first + p * kLlRowsPerPass + r0;
@@ -59,8 +62,8 @@ __global__ __launch_bounds__(kThreads) void lossless_fp4_to_fp8_kernel(const uin
     }
 
     __syncthreads();
-    // Block maxima.  Along a row: the 16 lanes of a tile row are one DPP row, so the lanes that share an output block
-    // reduce without LDS.  Down the rows: a lane folds its own consecutive rows while they stay in one block, and
+    // Block maxima.  Along a row: 16 lanes (one DPP row) cover 128 columns, the widest output block, so the lanes that
+    // share an output block reduce without LDS.  Down the rows: a lane folds its own consecutive rows while they stay in one block, and
     // only then does the first lane of each group touch the LDS table (16 atomics per 128 x 128 block, not 2048).
     uint32_t run = 0u;
 #pragma unroll
@@ -97,7 +100,7 @@ __global__ __launch_bounds__(kThreads) void lossless_fp4_to_fp8_kernel(const uin
         st_stream8(out + (int64_t)row * K + col, pack_e4m3x8<false>(v));
     }
 
-    for (int i = threadIdx.x; i < brows * bcols; i += kThreads) {
+    for (int i = threadIdx.x; i < brows * bcols; i += kLlThreads) {
         const int bm_i = i >> bcols_sh, bk_i = i & (bcols - 1);
         const int m = tile_m * brows + bm_i, k = tile_k * bcols + bk_i;
         if (m < out_nm && k < out_nk) {
@@ -145,9 +148,9 @@ extern "C" int tk_per_block_cast_lossless(const void *x, int64_t M, int64_t K, c
     const int rc = tk_check_per_block_cast_lossless(x, M, K, x_sf, x_sf_ld, x_sf_layout, x_bm, x_bk, out, out_sf, out_sf_ld,
                                                     out_sf_layout, out_bm, out_bk);
     if (rc != TK_OK || M == 0) return rc;
-    const dim3 grid((unsigned)((K + kLlTile - 1) / kLlTile), (unsigned)((M + kLlTile - 1) / kLlTile));
+    const dim3 grid((unsigned)((K + kLlTileK - 1) / kLlTileK), (unsigned)((M + kLlTile - 1) / kLlTile));
     auto log2i = [](int v) { int s = 0; while ((1 << s) < v) ++s; return s; };
-    hipLaunchKernelGGL(lossless_fp4_to_fp8_kernel, grid, dim3(kThreads), 0, static_cast<hipStream_t>(stream),
+    hipLaunchKernelGGL(lossless_fp4_to_fp8_kernel, grid, dim3(kLlThreads), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint8_t *>(x), const_cast<void *>(x_sf), x_sf_ld, (int)M, (int)K, x_sf_layout, log2i(x_bm), log2i(x_bk),
                        log2i(out_bm), log2i(out_bk), static_cast<uint8_t *>(out), out_sf, out_sf_ld, out_sf_layout, (int)((M + x_bm - 1) / x_bm),
                        (int)((K + x_bk - 1) / x_bk), (int)((M + out_bm - 1) / out_bm), (int)((K + out_bk - 1) / out_bk));
