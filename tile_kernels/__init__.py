@@ -1,9 +1,9 @@
 """Import-path alias: ``import tile_kernels`` resolves to the MI355X implementation.
 
 Code written against the reference's ``tile_kernels.quant`` / ``tile_kernels.config`` /
-``tile_kernels.testing`` finds the same names here.  Only the quantisation path and the two MoE
-layout helpers next to it exist; the other sub-packages of the reference (engram, mhc, transpose,
-modeling, torch, the rest of moe) are not provided.
+``tile_kernels.testing`` finds the same names here.  The quantisation package and the MoE layout
+helpers next to it (mapping, expansion, weighted reduction) exist; the other sub-packages of the
+reference (engram, mhc, transpose, modeling, torch, the rest of moe) are not provided.
 """
 import sys
 
@@ -15,5 +15,5 @@ for _name in ('config', 'moe', 'quant', 'testing', 'utils'):
     sys.modules[f'{__name__}.{_name}'] = getattr(_impl, _name)
 for _name in ('common', 'types'):
     sys.modules[f'{__name__}.quant.{_name}'] = sys.modules[f'tilekernels_amd.quant.{_name}']
-for _name in ('numeric', 'quant', 'generator'):
+for _name in ('numeric', 'quant', 'generator', 'bench'):
     sys.modules[f'{__name__}.testing.{_name}'] = sys.modules[f'tilekernels_amd.testing.{_name}']

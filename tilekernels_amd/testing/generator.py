@@ -59,6 +59,33 @@ def generate_topk_idx(params: dict, device='cuda') -> torch.Tensor:
     return topk_idx[~away.all(dim=1)].contiguous()
 
 
+# E5M6 keeps the top 12 bits of an fp16: its subnormals are k * 2^-20 for k = 1 .. 63, its smallest normal is 2^-14
+E5M6_SPECIAL_VALUES = (2.0 ** -20, 2.0 ** -14 * 63 / 64, 2.0 ** -14)
+
+
+def generate_e5m6_inputs(num_tokens: int, hidden: int, dtype: torch.dtype, device='cuda'):
+    """``(x, is_special)`` pairs for the E5M6 tests (tile_kernels/testing/generator.py:70-89): one random
+    tensor, then one constant tensor per special value whose last column holds 65024, so that the scale is 1
+    and the constant is cast as it stands."""
+    yield torch.randn((num_tokens, hidden), dtype=dtype, device=device), False
+    for value in E5M6_SPECIAL_VALUES:
+        x = torch.full((num_tokens, hidden), value, dtype=dtype, device=device)
+        x[:, -1] = 65024.0
+        yield x, True
+
+
+def generate_rand_float(shape, device='cuda') -> torch.Tensor:
+    """Normal values scaled by a power of two drawn uniformly from 2^-110 .. 2^126, non-finite values redrawn
+    and magnitudes capped at an eighth of the fp32 range (tile_kernels/testing/generator.py:92-105)."""
+    import random
+    x = torch.randn(shape, dtype=torch.float32, device=device) * float(2 ** random.randint(-110, 126))
+    bad = ~torch.isfinite(x)
+    if bad.any():
+        x[bad] = torch.randn((int(bad.sum()),), dtype=torch.float32, device=device)
+    cap = torch.finfo(torch.float32).max / 8
+    return x.clamp(-cap, cap)
+
+
 def generate_moe_layout(num_tokens: int, num_experts: int, num_topk: int, alignment: int, generator: torch.Generator,
                         drop_fraction: float = 0.0):
     """Expert-major expanded layout of a top-k routed batch, built on the CPU.
