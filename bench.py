@@ -228,7 +228,7 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_str
     value = w.bytes / (wall / steps) / 1e9
     achieved = w.bytes / (kern_us * 1e-6) / 1e9
     line = {
-        'metric': 'HBM GB/s (% of MI355X peak) + us/call, fused SwiGLU+FP8 quant [8192,4096]' if cfg == 3 else f'HBM GB/s, config {cfg}',
+        'metric': 'HBM GB/s (% of MI355X peak) + \u00b5s/call, fused SwiGLU+FP8 quant [8192,4096]' if cfg == 3 else f'HBM GB/s, config {cfg}',
         'value': round(value, 1), 'unit': 'GB/s', 'n_gpus': 1, 'steps': steps, 'warmup': warmup,
         'ms_per_step': round(ms_per_step, 6), 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'f32', 'data': 'synthetic',
