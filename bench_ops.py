@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Kernel timings of the operators around the headline path, one JSON line per operator.
 
-    python bench_ops.py [--steps 2000] [--warmup 1000] [--only NAME]
+    python bench_ops.py [--steps 2000] [--warmup 1000] [--only NAME[,NAME...]]
 
 Companion of bench.py (which measures the headline workload and keeps the driver's contract): the
 same method -- C-ABI calls on preallocated device buffers, buffer sets rotated past the 256 MB
@@ -43,24 +43,27 @@ def _sets_needed(footprint: int) -> int:
     return min(16, max(3, -(-int(1.6 * LLC_BYTES) // max(footprint, 1))))
 
 
-def op_cast_back():
-    import tilekernels_amd as tk
-    from tilekernels_amd import _ffi
-    lib = _ffi.load()
-    M, K = 8192, 4096
-    x = torch.randn((M, K), device='cuda', dtype=torch.bfloat16)
-    codes, sf = tk.quant.per_token_cast(x, 'e4m3', num_per_channels=128)
-    out = torch.empty((M, K), device='cuda', dtype=torch.bfloat16)
-    stream = _ffi.current_stream(x.device)
+def op_cast_back(out_name='bf16'):
+    def make():
+        import tilekernels_amd as tk
+        from tilekernels_amd import _ffi
+        lib = _ffi.load()
+        M, K = 8192, 4096
+        x = torch.randn((M, K), device='cuda', dtype=torch.bfloat16)
+        codes, sf = tk.quant.per_token_cast(x, 'e4m3', num_per_channels=128)
+        out = torch.empty((M, K), device='cuda', dtype=torch.bfloat16 if out_name == 'bf16' else torch.float32)
+        out_dtype = _ffi.TK_BF16 if out_name == 'bf16' else _ffi.TK_F32
+        stream = _ffi.current_stream(x.device)
 
-    def launch():
-        rc = lib.tk_cast_back(codes.data_ptr(), 0, M, K, sf.data_ptr(), sf.stride(0), 0, 1, 128, out.data_ptr(), 0, stream)
-        assert rc == 0, rc
-    def cpu():
-        from oracle import torch_ref
-        xq = (codes.cpu(), sf.cpu())
-        return lambda: torch_ref.cast_back(xq, 'bf16', (1, 128))
-    return launch, nbytes(codes, sf, out), nbytes(codes, sf, out), cpu
+        def launch():
+            rc = lib.tk_cast_back(codes.data_ptr(), 0, M, K, sf.data_ptr(), sf.stride(0), 0, 1, 128, out.data_ptr(), out_dtype, stream)
+            assert rc == 0, rc
+        def cpu():
+            from oracle import torch_ref
+            xq = (codes.cpu(), sf.cpu())
+            return lambda: torch_ref.cast_back(xq, out_name, (1, 128))
+        return launch, nbytes(codes, sf, out), nbytes(codes, sf, out), cpu
+    return make
 
 
 def op_requant():
@@ -419,7 +422,8 @@ OPS = [
        'swiglu_forward_and_per_token_cast e4m3 1x128, MoE-expanded bf16 [R,4096] with mask and routing weights', op_swiglu_weighted),
     Op('expand_to_fused_with_sf', 'expand_to_fused_with_sf e4m3 [4096,4096] + 1x128 scales -> [R,4096], top-8 of 256 experts, pad 128',
        op_expand_to_fused_with_sf),
-    Op('cast_back', 'cast_back e4m3 1x128 -> bf16, [8192,4096]', op_cast_back),
+    Op('cast_back', 'cast_back e4m3 1x128 -> bf16, [8192,4096]', op_cast_back('bf16')),
+    Op('cast_back_fp32', 'cast_back e4m3 1x128 -> fp32, [8192,4096]', op_cast_back('fp32')),
     Op('per_token_cast_quantized', 'per_token_cast of (e4m3 1x128) input -> e2m1 1x32, [8192,4096]', op_requant),
     Op('get_fused_mapping', 'get_fused_mapping 4096 tokens, top-8 of 256 experts, pad 128', op_get_fused_mapping),
     Op('expand_to_fused', 'expand_to_fused bf16 [4096,4096] -> [R,4096], top-8 of 256 experts, pad 128', op_expand_to_fused),
@@ -494,7 +498,7 @@ def main():
         sys.exit('bench_ops.py needs a GPU')
     torch.cuda.set_device(0)
     for op in OPS:
-        if a.only and a.only != op.name:
+        if a.only and op.name not in a.only.split(','):
             continue
         print(json.dumps(run(op, a.steps, a.warmup, not a.no_cpu)), flush=True)
         torch.cuda.empty_cache()

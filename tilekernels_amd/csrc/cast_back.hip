@@ -1,9 +1,11 @@
 // Dequantisation of block-scaled E4M3 / packed E2M1 codes back to bf16 or fp32 for gfx950.
 //
 // out[m, k] = float(code[m, k]) * sf[m / bm, k / bk], one fp32 product, then (for bf16) one
-// round-to-nearest-even conversion (v_cvt_pk_bf16_f32).  Pure streaming: a lane takes 8 consecutive
-// codes (8 or 4 bytes), their shared scale, and writes 16 (bf16) or 32 (fp32) bytes; a workgroup
-// covers 2 rows x up to 4096 columns (row-major scales) or 8 rows x 512 columns.
+// round-to-nearest-even conversion (v_cvt_pk_bf16_f32).  Pure streaming: for bf16 a lane takes 8
+// consecutive codes (8 or 4 bytes), their shared scale, and writes 16 bytes; for fp32 it takes 4 codes
+// of two pieces 256 columns apart and writes 16 bytes of each, so that every store instruction of a
+// wave covers whole cache lines.  A workgroup covers 2 rows x up to 4096 columns (row-major scales) or
+// 8 rows x 512 columns.
 //
 // Reference semantics: tile_kernels/quant/cast_back_kernel.py:19-75 (kernel) and :77-143 (wrappers),
 // tile_kernels/torch/cast.py:40-59 (oracle).
@@ -35,24 +37,52 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_bac
     const bool col_ok = FULL || col < K;
     const int row0 = tile_m * ROWS + (WIDE ? 0 : wave * RPW);
 
-    Raw8<InT> raw[RPW];
+    if constexpr (OUT_F32) {
+        // fp32 output: 8 values are 32 bytes, two 16-byte stores.  Were they a lane's own piece, each store
+        // instruction would write every other 16 bytes of its cache lines (half lines: 49.8 us for 8192 x 4096
+        // E4M3).  So a lane takes 4 codes of two pieces instead, columns 4 * lane and 256 + 4 * lane of the strip,
+        // and each store instruction writes 1024 consecutive bytes.  Two lanes load the same piece; the
+        // second load is served by the same fetch.
+        const bool hi = lane & 1;
+        const int pcol = strip * kStripCols + (lane >> 1) * 8;
+        Raw8<InT> raw[RPW][2];
 #pragma unroll
-    for (int r = 0; r < RPW; ++r) {
-        const bool ok = col_ok && (FULL || row0 + r < M);
-        raw[r].load(elem_ptr<InT>(x, row0 + r, K, col), ok);
-        raw[r].s = ok ? sf_load(sf, (row0 + r) / bm, col / bk) : 0.0f;
-    }
+        for (int r = 0; r < RPW; ++r) {
 #pragma unroll
-    for (int r = 0; r < RPW; ++r) {
-        if (!(col_ok && (FULL || row0 + r < M))) continue;
-        float v[8];
-        raw[r].get(v);
-        const int64_t idx = (int64_t)(row0 + r) * K + col;
-        if (OUT_F32) {
-            u32x4 *o = reinterpret_cast<u32x4 *>(reinterpret_cast<float *>(out) + idx);
-            __builtin_nontemporal_store(u32x4{f2u(v[0]), f2u(v[1]), f2u(v[2]), f2u(v[3])}, o);
-            __builtin_nontemporal_store(u32x4{f2u(v[4]), f2u(v[5]), f2u(v[6]), f2u(v[7])}, o + 1);
-        } else {
+            for (int h = 0; h < 2; ++h) {
+                const int c = pcol + h * (kStripCols / 2);
+                const bool ok = (FULL || c < K) && (FULL || row0 + r < M);
+                raw[r][h].load(elem_ptr<InT>(x, row0 + r, K, c), ok);
+                raw[r][h].s = ok ? sf_load(sf, (row0 + r) / bm, c / bk) : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int c = pcol + h * (kStripCols / 2);
+                if (!((FULL || c < K) && (FULL || row0 + r < M))) continue;
+                float v[4];
+                raw[r][h].get4(v, hi);
+                const int64_t idx = (int64_t)(row0 + r) * K + c + (hi ? 4 : 0);
+                __builtin_nontemporal_store(u32x4{f2u(v[0]), f2u(v[1]), f2u(v[2]), f2u(v[3])},
+                                            reinterpret_cast<u32x4 *>(reinterpret_cast<float *>(out) + idx));
+            }
+        }
+    } else {
+        Raw8<InT> raw[RPW];
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            const bool ok = col_ok && (FULL || row0 + r < M);
+            raw[r].load(elem_ptr<InT>(x, row0 + r, K, col), ok);
+            raw[r].s = ok ? sf_load(sf, (row0 + r) / bm, col / bk) : 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            if (!(col_ok && (FULL || row0 + r < M))) continue;
+            float v[8];
+            raw[r].get(v);
+            const int64_t idx = (int64_t)(row0 + r) * K + col;
             u32x4 w;
             w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[0], v[1]}), bf16x2));
             w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[2], v[3]}), bf16x2));
@@ -85,6 +115,8 @@ static void launch_cast_back_2(const void *x, void *out, const void *sf, int64_t
 template <typename InT, bool OUT_F32>
 static hipError_t launch_cast_back(const void *x, void *out, const void *sf, int64_t sf_ld, int M, int K, int sf_layout,
                                    int bm, int bk, hipStream_t stream) {
+    // wide tiles with column-major scales are no faster (E4M3 [8192, 4096]) and slower with 32 x 32 blocks (20.9 us
+    // against 16.2 us): a 2-row tile then uses 8 bytes of each scale line it touches
     if (sf_layout == TK_SF_ROW_F32) launch_cast_back_2<InT, OUT_F32, true>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);
     else launch_cast_back_2<InT, OUT_F32, false>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);
     return hipGetLastError();

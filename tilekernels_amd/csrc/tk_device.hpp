@@ -134,6 +134,12 @@ template <> struct Raw8<e4m3in_t> {
         v[0] = a.x * s; v[1] = a.y * s; v[2] = b.x * s; v[3] = b.y * s;
         v[4] = c.x * s; v[5] = c.y * s; v[6] = d.x * s; v[7] = d.y * s;
     }
+    // codes 0..3 (hi = false) or 4..7 of the piece
+    __device__ __forceinline__ void get4(float (&v)[4], bool hi) const {
+        const int h = (int)(hi ? w.y : w.x);
+        const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8(h, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(h, true);
+        v[0] = a.x * s; v[1] = a.y * s; v[2] = b.x * s; v[3] = b.y * s;
+    }
 };
 template <> struct Raw8<e2m1in_t> {
     uint32_t w;
@@ -148,6 +154,11 @@ template <> struct Raw8<e2m1in_t> {
         const f32x2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3);
         v[0] = a.x * s; v[1] = a.y * s; v[2] = b.x * s; v[3] = b.y * s;
         v[4] = c.x * s; v[5] = c.y * s; v[6] = d.x * s; v[7] = d.y * s;
+    }
+    __device__ __forceinline__ void get4(float (&v)[4], bool hi) const {
+        const uint32_t h = hi ? w >> 16 : w;
+        const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(h, 1.0f, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(h, 1.0f, 1);
+        v[0] = a.x * s; v[1] = a.y * s; v[2] = b.x * s; v[3] = b.y * s;
     }
 };
 
@@ -175,6 +186,14 @@ template <> struct Raw8<e5m6in_t> {
         v[5] = e5m6_value((w.y << 12) | (w.z >> 20)) * s;
         v[6] = e5m6_value(w.z >> 8) * s;
         v[7] = e5m6_value(w.z << 4) * s;
+    }
+    // codes 0..3 are the first 48 bits of the string, codes 4..7 the last 48
+    __device__ __forceinline__ void get4(float (&v)[4], bool hi) const {
+        const uint32_t a = hi ? (w.y << 16) | (w.z >> 16) : w.x, b = hi ? w.z & 0xFFFFu : w.y >> 16;
+        v[0] = e5m6_value(a >> 16) * s;
+        v[1] = e5m6_value(a >> 4) * s;
+        v[2] = e5m6_value((a << 8) | (b >> 8)) * s;
+        v[3] = e5m6_value(b << 4) * s;
     }
 };
 
@@ -383,10 +402,18 @@ struct SfRef {
 };
 
 __device__ __forceinline__ float sf_load(const SfRef &s, int m, int k) {
-    if (s.layout == TK_SF_ROW_F32) return reinterpret_cast<const float *>(s.base)[(int64_t)m * s.ld + k];
-    if (s.layout == TK_SF_COL_F32) return reinterpret_cast<const float *>(s.base)[(int64_t)k * s.ld + m];
-    const uint32_t e = reinterpret_cast<const uint8_t *>(s.base)[(int64_t)(k >> 2) * s.ld + 4 * (int64_t)m + (k & 3)];
-    return u2f(e << 23);
+    // Only the load sits inside the branches.  Arithmetic on the loaded value in there (the byte of the packed
+    // layout shifted into an exponent) makes the compiler wait for the load before it leaves the branch, and the
+    // loads of several rows then complete one after the other: dequantisation of E4M3 [8192, 4096] with packed
+    // scales took 19.2 us against 17.2 us with fp32 scales.  So the packed layout reads the aligned word that
+    // holds the byte, and the extraction happens after the branches with operands that are the identity for fp32.
+    const bool packed = s.layout == TK_SF_COL_UE8M0;
+    uint32_t w;
+    if (s.layout == TK_SF_ROW_F32) w = reinterpret_cast<const uint32_t *>(s.base)[(int64_t)m * s.ld + k];
+    else if (s.layout == TK_SF_COL_F32) w = reinterpret_cast<const uint32_t *>(s.base)[(int64_t)k * s.ld + m];
+    else w = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint8_t *>(s.base) + (int64_t)(k >> 2) * s.ld + 4 * (int64_t)m);
+    const uint32_t down = packed ? 8u * (uint32_t)(k & 3) : 0u, keep = packed ? 0xFFu : 0xFFFFFFFFu, up = packed ? 23u : 0u;
+    return u2f(((w >> down) & keep) << up);
 }
 
 // The same without a branch: the layout only selects how the byte offset is formed, and the packed layout
