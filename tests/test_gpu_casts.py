@@ -35,7 +35,7 @@ def _rand(shape, dtype, outliers=True):
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32], ids=['bf16', 'f32'])
 @pytest.mark.parametrize('M,K,N', [
     (401, 7168, 128), (401, 7168, 32), (37, 576, 128), (37, 576, 64), (37, 576, 32), (37, 576, 16), (37, 576, 576),
-    (1, 128, 128), (5, 64, 64), (16, 2048, 2048), (130, 2560, 128), (19, 3072, 3072), (64, 512, 128), (3, 4096, 16),
+    (1, 128, 128), (5, 64, 64), (16, 2048, 2048), (130, 2560, 128), (19, 3072, 3072), (64, 512, 128), (3, 4096, 16), (70, 5632, 128), (70, 6656, 32),
 ])
 def test_per_token_cast(M, K, N, dtype, fmt, mode):
     tk = _tk()

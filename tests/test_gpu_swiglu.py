@@ -47,7 +47,8 @@ def check_fused(got, want, nk, packed, what=''):
                          ids=lambda m: 'col%d-round%d-packed%d' % tuple(int(v) for v in m))
 @pytest.mark.parametrize('with_weights', [False, True])
 @pytest.mark.parametrize('with_mask', [False, True])
-@pytest.mark.parametrize('H,N', [(2048, 128), (288 * 4 + 128, 128), (1024, 1024), (3584, 128), (384, 384)])
+@pytest.mark.parametrize('H,N', [(2048, 128), (288 * 4 + 128, 128), (1024, 1024), (3584, 128), (384, 384),
+                                 (512, 128), (896, 128), (5632, 128)])   # one, two and eleven 512-column strips
 def test_swiglu_forward_and_per_token_cast(H, N, with_mask, with_weights, mode, clamp):
     tk = _tk()
     col, rnd, packed = mode

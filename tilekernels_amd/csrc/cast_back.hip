@@ -117,7 +117,7 @@ static hipError_t launch_cast_back(const void *x, void *out, const void *sf, int
                                    int bm, int bk, hipStream_t stream) {
     // wide tiles with column-major scales are no faster (E4M3 [8192, 4096]) and slower with 32 x 32 blocks (20.9 us
     // against 16.2 us): a 2-row tile then uses 8 bytes of each scale line it touches
-    if (sf_layout == TK_SF_ROW_F32) launch_cast_back_2<InT, OUT_F32, true>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);
+    if (sf_layout == TK_SF_ROW_F32 && wide_tiles_pay(K)) launch_cast_back_2<InT, OUT_F32, true>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);
     else launch_cast_back_2<InT, OUT_F32, false>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);
     return hipGetLastError();
 }

@@ -47,8 +47,8 @@ struct PerTokenParams {
 // Tile shapes (RPW = rows per wave):
 //   WIDE  (row-major scales):      RPW rows x (W*512) columns, W = blockDim.x/64 waves side by side on the same rows;
 //         the tile's scales are RPW contiguous runs, staged in LDS and stored as whole segments
-//   !WIDE (column-major layouts):  4*RPW rows x 512 columns, the 4 waves stacked; the staged scales
-//         are stored transposed, 4*RPW rows per contiguous segment
+//   !WIDE (column-major layouts, and rows of at most 1024 columns):  4*RPW rows x 512 columns, the 4 waves stacked;
+//         the staged scales are stored transposed, 4*RPW rows per contiguous segment (row-major: one short run per row)
 // FULL: the tile grid covers the matrix exactly, so no bounds checks are compiled in.
 template <typename InT, int G, int FMT, int RPW, bool WIDE, bool FULL>
 __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_token_cast_kernel(TK_PT_KERNEL_ARGS) {
@@ -130,6 +130,7 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
     if (p.mode != TK_CAST_GIVEN_SF) {
         __syncthreads();
         if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
+        else if (p.sf.layout == TK_SF_ROW_F32) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, GPS, tile_m * ROWS, tile_k * GPS);
         else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
     }
 }
@@ -242,7 +243,7 @@ static void launch_per_token_tiled(PerTokenParams &p, hipStream_t stream) {
 template <typename InT, int G, int FMT>
 static void launch_per_token_group(PerTokenParams &p, hipStream_t stream) {
     // a caller-supplied scale tensor is only read, so either tile shape does
-    if (p.sf.layout == TK_SF_ROW_F32) launch_per_token_tiled<InT, G, FMT, true>(p, stream);
+    if (p.sf.layout == TK_SF_ROW_F32 && wide_tiles_pay(p.K)) launch_per_token_tiled<InT, G, FMT, true>(p, stream);
     else launch_per_token_tiled<InT, G, FMT, false>(p, stream);
 }
 

@@ -91,7 +91,8 @@ __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
 //             contiguous run: no LDS stage and no workgroup barrier at the end of the tile
 //   T_WIDE    (row-major scales, other H): RPW rows x (W*512) columns, W waves side by side; the tile's scales are
 //             RPW contiguous runs, staged in LDS and stored as whole segments
-//   T_STACKED (column-major layouts): 4*RPW rows x 512 columns, the 4 waves stacked, scales stored transposed
+//   T_STACKED (column-major layouts, and H <= 1024): 4*RPW rows x 512 columns, the 4 waves stacked, scales stored
+//             transposed (row-major: one short run per row)
 // W = blockDim.x / 64.  FULL: the tile grid covers the matrix exactly: no bounds checks are compiled in.
 // MASK: pos_to_expert is given.
 enum { T_STACKED = 0, T_WIDE = 1, T_ROW = 2 };
@@ -223,6 +224,7 @@ __global__ __launch_bounds__(TILE != T_STACKED ? 64 * kMaxWideWaves : kThreads) 
         if constexpr (!ROW) {
             __syncthreads();
             if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
+            else if (p.sf.layout == TK_SF_ROW_F32) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, GPS, tile_m * ROWS, tile_k * GPS);
             else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
             if (LOOP && (int)gridDim.x < total) __syncthreads();   // stage is reused by the next tile
         }
@@ -324,7 +326,7 @@ static hipError_t launch_swiglu_2(SwigluParams &p, bool row_group, int max_block
     if (row_group) {
         const int grid = max_blocks > 0 && max_blocks < p.R ? max_blocks : p.R;
         hipLaunchKernelGGL((swiglu_rowgroup_kernel<InT, CLAMP>), dim3(grid), dim3(kThreads), 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
-    } else if (p.sf.layout != TK_SF_ROW_F32) {
+    } else if (p.sf.layout != TK_SF_ROW_F32 || !wide_tiles_pay(p.H)) {
         launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, T_STACKED>(p, max_blocks, stream);
     } else if (p.H % (kSwigluRowsPerWave * kStripCols) == 0) {
         launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, T_ROW>(p, max_blocks, stream);

@@ -16,12 +16,18 @@ constexpr int kWaves = kThreads / 64;
 constexpr int kMaxWideWaves = 8;
 
 // Number of waves of a wide tile (waves side by side, 512 columns each) for a row of `strips`
-// 512-column strips: the largest of 8..3 that divides it, so that no wave idles; 4 if none does.
+// 512-column strips: the largest of 8..3 that divides it, so that no wave idles; 0 if none does.
 inline int wide_tile_waves(int strips) {
     for (int w = kMaxWideWaves; w >= 3; --w)
         if (strips % w == 0) return w;
-    return 4;
+    return 0;
 }
+
+// Wide tiles are for rows whose strips split evenly over 3..8 waves.  Other rows take stacked tiles: one or two
+// strips would leave most waves of a wide tile without columns (SwiGLU of bf16 [65536, 2 x 512]: 62 us wide, 27 us
+// stacked), and 11 or 13 strips still idle one wave of a tile in 12 or 14 (per-token cast of bf16 [20096, 6656]:
+// 62.7 us wide with 7 waves, 57.4 us stacked).
+inline bool wide_tiles_pay(int64_t cols) { return wide_tile_waves((int)((cols + kStripCols - 1) / kStripCols)) != 0; }
 
 struct bf16_t { uint16_t bits; };
 struct e4m3in_t {};   // input that is itself E4M3 codes with block scales
