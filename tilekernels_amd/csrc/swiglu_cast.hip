@@ -91,33 +91,38 @@ __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
 //             contiguous run: no LDS stage and no workgroup barrier at the end of the tile
 //   T_WIDE    (row-major scales, other H): RPW rows x (W*512) columns, W waves side by side; the tile's scales are
 //             RPW contiguous runs, staged in LDS and stored as whole segments
-//   T_STACKED (column-major layouts, and H <= 1024): 4*RPW rows x 512 columns, the 4 waves stacked, scales stored
+//   T_ROWC    (column-major layouts, H a multiple of RPW*512): the same 4 rows x (RPW*512) columns, one row per wave; the
+//             scales are staged in LDS and stored transposed, 4 rows per run.  Against stacked tiles, whose waves
+//             read 1 KB from each of 8 row halves instead of 4 KB from 2 (us per call, bf16, packed scales):
+//             [32768, 2 x 2048] 60.6 -> 52.4, [16384, 2 x 4096] 69.4 -> 53.9, [8192, 2 x 6144] 48.8 -> 40.9
+//   T_STACKED (other H with column-major layouts, and rows that do not split evenly over the waves of a wide tile): 4*RPW rows x 512 columns, the 4 waves stacked, scales stored
 //             transposed (row-major: one short run per row)
 // W = blockDim.x / 64.  FULL: the tile grid covers the matrix exactly: no bounds checks are compiled in.
 // MASK: pos_to_expert is given.
-enum { T_STACKED = 0, T_WIDE = 1, T_ROW = 2 };
+enum { T_STACKED = 0, T_WIDE = 1, T_ROW = 2, T_ROWC = 3 };
 
 template <typename InT, int CLAMP, int RPW, int TILE, bool FULL, bool MASK>
-__global__ __launch_bounds__(TILE != T_STACKED ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
+__global__ __launch_bounds__(TILE == T_WIDE || TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
     TK_SWIGLU_KERNEL_UNPACK;
-    constexpr bool WIDE = TILE == T_WIDE, ROW = TILE == T_ROW;
+    constexpr bool WIDE = TILE == T_WIDE, ROWC = TILE == T_ROWC, ROW = TILE == T_ROW || ROWC;   // ROW: a wave's pieces lie along one row
+    constexpr bool DIRECT = TILE == T_ROW;  // the wave stores its scales itself
     constexpr int GPS = kStripCols / 128;   // 4 groups per strip
-    constexpr int ROWS = WIDE ? RPW : kWaves * RPW;          // rows per tile (T_ROW: blockDim.x / 64, not used as a constant)
-    constexpr int SGPR = WIDE ? kMaxWideWaves * GPS : GPS;   // staged groups per row (capacity)
+    constexpr int ROWS = WIDE ? RPW : (ROWC ? kWaves : kWaves * RPW);   // rows per tile (T_ROW: blockDim.x / 64, not used as a constant)
+    constexpr int SGPR = WIDE ? kMaxWideWaves * GPS : (ROWC ? RPW * GPS : GPS);   // staged groups per row (capacity)
     // The counting variant loops over tiles (its grid is capped so that few workgroups touch the global
     // counters); every other variant has one workgroup per tile on a 2-D grid, which keeps integer
     // divisions and further kernel-argument loads out of the path to the first memory load.
     constexpr bool LOOP = CLAMP == 2;
-    const int nwaves = TILE != T_STACKED ? p.nwaves : kWaves;
-    const int rows = ROW ? nwaves : ROWS;
+    const int nwaves = (WIDE || DIRECT) ? p.nwaves : kWaves;
+    const int rows = DIRECT ? nwaves : ROWS;
     using RS = RowScales<448, RPW, 16>;
-    __shared__ uint32_t stage[ROW ? 1 : ROWS][ROW ? 1 : SGPR];
+    __shared__ uint32_t stage[DIRECT ? 1 : ROWS][DIRECT ? 1 : SGPR];
 
     const int total = LOOP ? ((p.R + rows - 1) / rows) * p.tiles_k : 1;
     const int lane = threadIdx.x & 63, wave = wave_id();
     const bool has_weight = p.pos_to_token_topk != nullptr;
     const int own = lane & 15;
-    const int srow = WIDE ? 0 : wave * RPW;
+    const int srow = WIDE ? 0 : (ROWC ? wave : wave * RPW);
     ClampCounter<CLAMP> counter;
 
     for (int tile = LOOP ? (int)blockIdx.x : 0; tile < total; tile += LOOP ? (int)gridDim.x : 1) {
@@ -205,7 +210,9 @@ __global__ __launch_bounds__(TILE != T_STACKED ? 64 * kMaxWideWaves : kThreads) 
         if (own < RS::A) {
 #pragma unroll
             for (int c = 0; c < RS::NC; ++c) {
-                if constexpr (ROW) {
+                if constexpr (ROWC) {
+                    stage[srow][(c * RS::A + own) * GPS + (lane >> 4)] = p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
+                } else if constexpr (DIRECT) {
                     // group (lane >> 4) of piece c*A + own: the wave's scales form one run of RPW * 4 floats
                     const int k = (strip + c * RS::A + own) * GPS + (lane >> 4);
                     if (FULL || (row0 < p.R && k < p.sf.nk))
@@ -221,9 +228,10 @@ __global__ __launch_bounds__(TILE != T_STACKED ? 64 * kMaxWideWaves : kThreads) 
             if ((FULL || col + r * kColStep < p.H) && (FULL || row0 + r * kRowStep < p.R))
                 quantise_store8<TK_E4M3, false>(v[r], rs.inv[r], p.out + (int64_t)(row0 + r * kRowStep) * p.H, col + r * kColStep);
         TK_TRACE(2);
-        if constexpr (!ROW) {
+        if constexpr (!DIRECT) {
             __syncthreads();
-            if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
+            if (ROWC) sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
+            else if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
             else if (p.sf.layout == TK_SF_ROW_F32) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, GPS, tile_m * ROWS, tile_k * GPS);
             else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
             if (LOOP && (int)gridDim.x < total) __syncthreads();   // stage is reused by the next tile
@@ -302,8 +310,8 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
     // masked: 1: 14.9 / 61.6, 2: 14.85 / 62.1, 4: 14.68 / 62.9, 8: 15.15 / 63.4.  A masked batch is better off with
     // single-wave workgroups: a wave whose row is padding is done at once and frees its slot alone.
     const int waves = TILE == T_WIDE ? wide_tile_waves(strips) : (TILE == T_ROW && p.pos_to_expert ? 1 : kWaves);
-    const int rows = TILE == T_WIDE ? RPW : (TILE == T_ROW ? waves : kWaves * RPW);
-    const int cols = TILE == T_WIDE ? waves * kStripCols : (TILE == T_ROW ? RPW * kStripCols : kStripCols);
+    const int rows = TILE == T_WIDE ? RPW : (TILE == T_ROW || TILE == T_ROWC ? waves : kWaves * RPW);
+    const int cols = TILE == T_WIDE ? waves * kStripCols : (TILE == T_ROW || TILE == T_ROWC ? RPW * kStripCols : kStripCols);
     const int tiles_m = (p.R + rows - 1) / rows;
     p.tiles_k = (p.H + cols - 1) / cols;
     p.nwaves = waves;
@@ -326,6 +334,10 @@ static hipError_t launch_swiglu_2(SwigluParams &p, bool row_group, int max_block
     if (row_group) {
         const int grid = max_blocks > 0 && max_blocks < p.R ? max_blocks : p.R;
         hipLaunchKernelGGL((swiglu_rowgroup_kernel<InT, CLAMP>), dim3(grid), dim3(kThreads), 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+    } else if (p.sf.layout != TK_SF_ROW_F32 && p.H % (kSwigluRowsPerWave * kStripCols) == 0) {
+        // (other H, where the last column tile of a row is partly empty and the loads are bounds-checked, are
+        // better off with stacked tiles: [16384, 2 x 2560] 35.6 us stacked, 44.2 us this way)
+        launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, T_ROWC>(p, max_blocks, stream);
     } else if (p.sf.layout != TK_SF_ROW_F32 || !wide_tiles_pay(p.H)) {
         launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, T_STACKED>(p, max_blocks, stream);
     } else if (p.H % (kSwigluRowsPerWave * kStripCols) == 0) {
