@@ -27,10 +27,11 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_bac
                                                                                          int nm, int nk) {
     constexpr int RPW = kBackRowsPerWave, ROWS = WIDE ? RPW : kWaves * RPW;
     const SfRef sf{a_sf, a_sf_ld, a_sf_layout, nm, nk};
-    // geom: wide tiles: waves per tile, the tile index comes from a 2-D grid (x = row tile, y = column
+    // geom: wide tiles: waves per tile, the tile index comes from the grid (x = column tile, y and z = row
     // tile); otherwise the number of column tiles of a 1-D grid
-    const int tile_m = WIDE ? (int)blockIdx.x : (int)blockIdx.x / geom;
-    const int tile_k = WIDE ? (int)blockIdx.y : (int)blockIdx.x - tile_m * geom;
+    const bool one_col = geom * kStripCols >= K;   // wide tiles: the waves of one tile cover a whole row
+    const int tile_m = WIDE ? tile_grid_row(one_col) : (int)blockIdx.x / geom;
+    const int tile_k = WIDE ? tile_grid_col(one_col) : (int)blockIdx.x - tile_m * geom;
     const int lane = threadIdx.x & 63, wave = wave_id();
     const int strip = WIDE ? tile_k * geom + wave : tile_k;
     const int col = strip * kStripCols + lane * 8;
@@ -103,10 +104,10 @@ static void launch_cast_back_2(const void *x, void *out, const void *sf, int64_t
     const int tiles_m = (M + rows - 1) / rows, tiles_k = (K + cols - 1) / cols;
     const int nm = (M + bm - 1) / bm, nk = (K + bk - 1) / bk;
     const dim3 block(64 * waves);
-    const dim3 grid = WIDE ? dim3((unsigned)tiles_m, (unsigned)tiles_k) : dim3((unsigned)(tiles_m * tiles_k));
+    const dim3 grid = WIDE ? tile_grid(tiles_k, tiles_m) : dim3((unsigned)(tiles_m * tiles_k));
     const int geom = WIDE ? waves : tiles_k;
     void *sfp = const_cast<void *>(sf);
-    if (M % rows == 0 && K % cols == 0)
+    if (M % rows == 0 && K % cols == 0 && (!WIDE || tile_grid_exact(tiles_k, tiles_m)))
         hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, true>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, geom, bm, bk, sf_layout, nm, nk);
     else
         hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, false>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, geom, bm, bk, sf_layout, nm, nk);
@@ -142,7 +143,6 @@ extern "C" int tk_check_cast_back(const void *x, int x_fmt, int64_t M, int64_t K
     const int64_t need = x_sf_layout == TK_SF_ROW_F32 ? nk : (x_sf_layout == TK_SF_COL_F32 ? nm : 4 * nm);
     if (x_sf_ld < need) return TK_ERR_BAD_STRIDE;
     if (((M + 1) / 2) * ((K + kStripCols - 1) / kStripCols) > INT32_MAX - 8) return TK_ERR_TOO_LARGE;
-    if (K / (3 * kStripCols) > 65535) return TK_ERR_TOO_LARGE;   // column tiles of the wide layout ride on grid.y
     return TK_OK;
 }
 

@@ -22,7 +22,7 @@ struct PerTokenParams {
     SfRef sf;
     int64_t x_ld;     // (logical) elements between rows of x
     int M, K;
-    int geom;         // wide tiles: waves per tile (2-D grid: x = row tile, y = column tile); else column tiles (1-D grid)
+    int geom;         // wide tiles: waves per tile (grid: x = column tile, y and z = row tile); else column tiles (1-D grid)
     int round_sf, mode;
     SfRef xsf;        // quantised input only: its block scales ...
     int in_bm, in_bk; // ... and their block shape
@@ -62,8 +62,9 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
     using RS = RowScales<Fmt<FMT>::qmax, RPW, LPG>;
     __shared__ uint32_t stage[ROWS][SGPR];
 
-    const int tile_m = WIDE ? (int)blockIdx.x : (int)blockIdx.x / p.geom;
-    const int tile_k = WIDE ? (int)blockIdx.y : (int)blockIdx.x - tile_m * p.geom;
+    const bool one_col = p.geom * kStripCols >= p.K;   // wide tiles: the waves of one tile cover a whole row
+    const int tile_m = WIDE ? tile_grid_row(one_col) : (int)blockIdx.x / p.geom;
+    const int tile_k = WIDE ? tile_grid_col(one_col) : (int)blockIdx.x - tile_m * p.geom;
     const int lane = threadIdx.x & 63, wave = wave_id();
     const int strip = WIDE ? tile_k * nwaves + wave : tile_k;
     const int col = strip * kStripCols + lane * 8;
@@ -233,8 +234,8 @@ static void launch_per_token_tiled(PerTokenParams &p, hipStream_t stream) {
     const int tiles_m = (p.M + rows - 1) / rows, tiles_k = (p.K + cols - 1) / cols;
     p.geom = WIDE ? waves : tiles_k;
     const dim3 block(64 * waves);
-    const dim3 grid = WIDE ? dim3((unsigned)tiles_m, (unsigned)tiles_k) : dim3((unsigned)(tiles_m * tiles_k));
-    if (p.M % rows == 0 && p.K % cols == 0)
+    const dim3 grid = WIDE ? tile_grid(tiles_k, tiles_m) : dim3((unsigned)(tiles_m * tiles_k));
+    if (p.M % rows == 0 && p.K % cols == 0 && (!WIDE || tile_grid_exact(tiles_k, tiles_m)))
         hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, true>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
     else
         hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, false>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
@@ -300,7 +301,6 @@ extern "C" int tk_check_per_token_cast(const void *x, int x_dtype, int64_t M, in
     const int64_t nk = (K + group - 1) / group;
     if (M * nk > INT32_MAX) return TK_ERR_TOO_LARGE;
     if (((M + 3) / 4) * ((K + kStripCols - 1) / kStripCols) > INT32_MAX) return TK_ERR_TOO_LARGE;   // tile count
-    if (K / (3 * kStripCols) > 65535) return TK_ERR_TOO_LARGE;                                      // column tiles ride on grid.y
     const int64_t need = sf_layout == TK_SF_ROW_F32 ? nk : (sf_layout == TK_SF_COL_F32 ? M : 4 * M);
     if (sf_ld < need) return TK_ERR_BAD_STRIDE;
     if (sf_layout == TK_SF_COL_UE8M0 && sf_ld % 4 != 0) return TK_ERR_MISALIGNED;
@@ -367,7 +367,6 @@ extern "C" int tk_check_per_token_cast_quantized(const void *x, int x_fmt, int64
     const int64_t xnm = (M + x_bm - 1) / x_bm, xnk = (K + x_bk - 1) / x_bk;
     const int64_t xneed = x_sf_layout == TK_SF_ROW_F32 ? xnk : (x_sf_layout == TK_SF_COL_F32 ? xnm : 4 * xnm);
     if (x_sf_ld < xneed) return TK_ERR_BAD_STRIDE;
-    if (K / (3 * kStripCols) > 65535) return TK_ERR_TOO_LARGE;   // column tiles ride on grid.y
     return TK_OK;
 }
 

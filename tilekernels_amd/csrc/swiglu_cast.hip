@@ -101,7 +101,8 @@ __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
 // MASK: pos_to_expert is given.
 enum { T_STACKED = 0, T_WIDE = 1, T_ROW = 2, T_ROWC = 3 };
 
-template <typename InT, int CLAMP, int RPW, int TILE, bool FULL, bool MASK>
+// ONECOL: the grid is known to be a single column of tiles (else it is found out at run time)
+template <typename InT, int CLAMP, int RPW, int TILE, bool FULL, bool MASK, bool ONECOL>
 __global__ __launch_bounds__(TILE == T_WIDE || TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
     TK_SWIGLU_KERNEL_UNPACK;
     constexpr bool WIDE = TILE == T_WIDE, ROWC = TILE == T_ROWC, ROW = TILE == T_ROW || ROWC;   // ROW: a wave's pieces lie along one row
@@ -126,8 +127,8 @@ __global__ __launch_bounds__(TILE == T_WIDE || TILE == T_ROW ? 64 * kMaxWideWave
     ClampCounter<CLAMP> counter;
 
     for (int tile = LOOP ? (int)blockIdx.x : 0; tile < total; tile += LOOP ? (int)gridDim.x : 1) {
-        const int tile_m = LOOP ? tile / p.tiles_k : (int)blockIdx.x;
-        const int tile_k = LOOP ? tile - tile_m * p.tiles_k : (int)blockIdx.y;
+        const int tile_m = LOOP ? tile / p.tiles_k : tile_grid_row(ONECOL || p.tiles_k == 1);
+        const int tile_k = LOOP ? tile - tile_m * p.tiles_k : tile_grid_col(ONECOL || p.tiles_k == 1);
         // piece r of the wave: row `row0 + (ROW ? 0 : r)`, columns from `col + (ROW ? r * 512 : 0)`
         const int strip = ROW ? tile_k * RPW : (WIDE ? tile_k * nwaves + wave : tile_k);
         const int col = strip * kStripCols + lane * 8;
@@ -154,14 +155,15 @@ __global__ __launch_bounds__(TILE == T_WIDE || TILE == T_ROW ? 64 * kMaxWideWave
             if (FULL && !MASK) {
                 rg[r].load(xr);
                 ru[r].load(xr + p.H);
-            } else if (FULL && MASK && TK_MASK_BRANCHLESS) {
+            } else if (TK_MASK_BRANCHLESS) {
                 // no branch around the loads (a branch would make the compiler wait for all eight loads
-                // before the first row is evaluated): a padding row reads the first bytes of the matrix,
-                // which every wave shares, and is cleared by value
-                const InT *src = live[r] ? xr : reinterpret_cast<const InT *>(p.x);
+                // before the first row is evaluated): a padding row, and a lane beyond the last row or column,
+                // reads the first bytes of the matrix, which every wave shares, and is cleared by value
+                const bool ok = live[r] && piece_ok;
+                const InT *src = ok ? xr : reinterpret_cast<const InT *>(p.x);
                 rg[r].load(src);
-                ru[r].load(live[r] ? xr + p.H : src);
-                if (!live[r]) { rg[r].zero(); ru[r].zero(); }
+                ru[r].load(ok ? xr + p.H : src);
+                if (!ok) { rg[r].zero(); ru[r].zero(); }
             } else {
                 rg[r].load(xr, live[r] && piece_ok);
                 ru[r].load(xr + p.H, live[r] && piece_ok);
@@ -318,15 +320,29 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
     const int total = tiles_m * p.tiles_k;
     const dim3 block(64 * waves);
     const dim3 grid = CLAMP == 2 ? dim3((unsigned)((max_blocks > 0 && max_blocks < total) ? max_blocks : total))
-                                 : dim3((unsigned)tiles_m, (unsigned)p.tiles_k);
-    const bool full = p.R % rows == 0 && p.H % cols == 0;
+                                 : tile_grid(p.tiles_k, tiles_m);
+    const bool full = p.R % rows == 0 && p.H % cols == 0 && (CLAMP == 2 || tile_grid_exact(p.tiles_k, tiles_m));
+    // the row-wise tiles of the common widths (H = 2048: one column of tiles) get a kernel of their own: the
+    // run-time test costs the [8192, 2 x 2048] call 0.2 us
+    constexpr bool ROWWISE = TILE == T_ROW || TILE == T_ROWC;
+    const bool onecol = ROWWISE && p.tiles_k == 1;
+#define TK_SWIGLU_LAUNCH(FULL_, MASK_)                                                                                          \
+    do {                                                                                                                        \
+        if (onecol)                                                                                                             \
+            hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, FULL_, MASK_, ROWWISE>), grid, block, 0, stream,      \
+                               TK_SWIGLU_LAUNCH_ARGS(p));                                                                       \
+        else                                                                                                                    \
+            hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, FULL_, MASK_, false>), grid, block, 0, stream,        \
+                               TK_SWIGLU_LAUNCH_ARGS(p));                                                                       \
+    } while (0)
     if (p.pos_to_expert) {
-        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, true, true>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
-        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, false, true>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+        if (full) TK_SWIGLU_LAUNCH(true, true);
+        else TK_SWIGLU_LAUNCH(false, true);
     } else {
-        if (full) hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, true, false>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
-        else hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, false, false>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+        if (full) TK_SWIGLU_LAUNCH(true, false);
+        else TK_SWIGLU_LAUNCH(false, false);
     }
+#undef TK_SWIGLU_LAUNCH
 }
 
 template <typename InT, int CLAMP>
@@ -388,7 +404,7 @@ extern "C" int tk_check_swiglu_per_token_cast(const void *x, int x_dtype, int64_
     if (sf_ld < need) return TK_ERR_BAD_STRIDE;
     if (sf_layout == TK_SF_COL_UE8M0 && sf_ld % 4 != 0) return TK_ERR_MISALIGNED;
     const int64_t tiles = ((R + 3) / 4) * ((H + kStripCols - 1) / kStripCols);
-    if (tiles > INT32_MAX - 8 || H / kStripCols > 65535) return TK_ERR_TOO_LARGE;   // grid.y carries the column tiles
+    if (tiles > INT32_MAX - 8) return TK_ERR_TOO_LARGE;
     return TK_OK;
 }
 
