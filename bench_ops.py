@@ -149,7 +149,7 @@ def op_swiglu_backward(group=128, rows=8192, hidden=2048):
         import tilekernels_amd as tk
         from tilekernels_amd import _ffi
         lib = _ffi.load()
-        R, H, T, K = rows, hidden, rows // 8, 8
+        R, H, T, K = rows, hidden, (rows + 7) // 8, 8
         x = torch.randn((R, 2 * H), device='cuda', dtype=torch.bfloat16)
         codes, sf = tk.quant.per_token_cast(x, 'e4m3', num_per_channels=group)
         del x
@@ -157,7 +157,9 @@ def op_swiglu_backward(group=128, rows=8192, hidden=2048):
         w = torch.rand((T, K), device='cuda')
         ptt = torch.randperm(T * K, device='cuda').to(torch.int32)
         t2p = torch.empty((T * K,), dtype=torch.int32, device='cuda')
-        t2p[ptt.long()] = torch.arange(R, dtype=torch.int32, device='cuda')
+        ptt = ptt[:R].contiguous()
+        t2p.fill_(-1)
+        t2p[ptt.long()] = torch.arange(R, dtype=torch.int32, device="cuda")
         out = torch.empty((R, H), device='cuda', dtype=torch.bfloat16)
         q = torch.empty((R, 2 * H), device='cuda', dtype=torch.float8_e4m3fn)
         q_sf = torch.empty((R, 2 * H // group), device='cuda', dtype=torch.float32)

@@ -52,9 +52,11 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_bac
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int c = pcol + h * (kStripCols / 2);
+                // no branch around the loads: a lane beyond the last row or column reads the first codes and the first
+                // scale, and writes nothing
                 const bool ok = (FULL || c < K) && (FULL || row0 + r < M);
-                raw[r][h].load(elem_ptr<InT>(x, row0 + r, K, c), ok);
-                raw[r][h].s = ok ? sf_load(sf, (row0 + r) / bm, c / bk) : 0.0f;
+                raw[r][h].load(ok ? elem_ptr<InT>(x, row0 + r, K, c) : x);
+                raw[r][h].s = sf_load(sf, ok ? (row0 + r) / bm : 0, ok ? c / bk : 0);
             }
         }
 #pragma unroll
@@ -75,8 +77,8 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_bac
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
             const bool ok = col_ok && (FULL || row0 + r < M);
-            raw[r].load(elem_ptr<InT>(x, row0 + r, K, col), ok);
-            raw[r].s = ok ? sf_load(sf, (row0 + r) / bm, col / bk) : 0.0f;
+            raw[r].load(ok ? elem_ptr<InT>(x, row0 + r, K, col) : x);
+            raw[r].s = sf_load(sf, ok ? (row0 + r) / bm : 0, ok ? col / bk : 0);
         }
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {

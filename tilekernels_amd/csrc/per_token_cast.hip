@@ -79,8 +79,15 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
         const void *xp = elem_ptr<InT>(p.x, row0 + r, p.x_ld, col);
-        if (FULL) raw[r].load(xp);
-        else raw[r].load(xp, col_ok && row0 + r < p.M);
+        if (FULL) {
+            raw[r].load(xp);
+        } else {
+            // no branch around the load (the loads of the wave's rows then go out together): a lane beyond the last
+            // row or column reads the first bytes of the matrix and is cleared by value
+            const bool ok = col_ok && row0 + r < p.M;
+            raw[r].load(ok ? xp : p.x);
+            if (!ok) raw[r].zero();
+        }
         if constexpr (Elem<InT>::quantised) {
             // the 8 codes of a lane share one input scale (input blocks are at least 32 columns wide)
             const bool ok = col_ok && (FULL || row0 + r < p.M);

@@ -179,6 +179,7 @@ template <> struct Raw8<e2m1in_t> {
         w = 0u;
         if (ok) load(p);
     }
+    __device__ __forceinline__ void zero() { w = 0u; s = 0.0f; }
     __device__ __forceinline__ void get(float (&v)[8]) const {
         const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1);
         const f32x2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3);
@@ -207,6 +208,7 @@ template <> struct Raw8<e5m6in_t> {
         w = u32x3{0u, 0u, 0u};
         if (ok) load(p);
     }
+    __device__ __forceinline__ void zero() { w = u32x3{0u, 0u, 0u}; s = 0.0f; }
     __device__ __forceinline__ void get(float (&v)[8]) const {
         v[0] = e5m6_value(w.x >> 16) * s;
         v[1] = e5m6_value(w.x >> 4) * s;
