@@ -52,7 +52,7 @@ def test_get_fused_mapping_no_tokens():
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32, torch.float8_e4m3fn])
-@pytest.mark.parametrize('hidden', [576, 2048, 7168])
+@pytest.mark.parametrize('hidden', [128, 576, 2048, 7168])
 @pytest.mark.parametrize('T,K,E', [(1001, 8, 64), (257, 2, 9), (3, 1, 4), (9, 3, 5)])
 def test_expand_to_fused(T, K, E, hidden, dtype):
     tk = _tk()

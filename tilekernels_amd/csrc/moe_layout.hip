@@ -197,6 +197,22 @@ constexpr int kExpandChunk = kThreads * 16;
 // 62 us with plain stores; pairs of 8-byte system-scope stores are several times slower still.
 __device__ __forceinline__ void expand_store16(void *p, u32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p)); }
 
+// Padding workgroup `pb` of the short-rows kernel: zero the rows among its pad_rows consecutive expanded rows that no
+// token maps to (the same loop as in the kernel for long rows, which keeps its own copy: sharing this function cost
+// that kernel 2 % with scale rows).
+__device__ __forceinline__ void expand_zero_padding(int pb, int pad_rows, int num_expanded, int64_t row_bytes, uint8_t *out,
+                                                    const int32_t *pos_to_expert, bool with_sf, int sf_cols, uint32_t *out_sf,
+                                                    int64_t out_sf_ld, int sf_col_major) {
+    const int r0 = pb * pad_rows;
+    for (int r = r0; r < r0 + pad_rows && r < num_expanded; ++r) {
+        if (uniform_load(pos_to_expert + r) >= 0) continue;
+        uint8_t *dst = out + (int64_t)r * row_bytes;
+        for (int64_t off = (int64_t)threadIdx.x * 16; off < row_bytes; off += kExpandChunk) expand_store16(dst + off, u32x4{0u, 0u, 0u, 0u});
+        if (with_sf)
+            for (int j = threadIdx.x; j < sf_cols; j += kThreads) out_sf[sf_col_major ? (int64_t)j * out_sf_ld + r : (int64_t)r * out_sf_ld + j] = 0u;
+    }
+}
+
 __global__ __launch_bounds__(kThreads) void expand_to_fused_kernel(const uint8_t *x, int64_t row_bytes, const int32_t *token_topk_to_pos,
                                                                    int num_topk, int chunks, int copy_blocks, int num_tokens,
                                                                    int num_expanded, uint8_t *out, const int32_t *pos_to_expert,
@@ -230,6 +246,39 @@ __global__ __launch_bounds__(kThreads) void expand_to_fused_kernel(const uint8_t
     }
 }
 
+// Rows of at most 2 KB (a kernel of its own: as a branch of the one above it cost that one 5 %).  The workgroup's
+// threads form kpw groups of tpr threads (tpr * 16 >= row_bytes), and group g copies the row to position kg * kpw + g
+// of the token, still one load and one store per thread.  (With one position per workgroup half or more of the
+// threads had nothing to copy: bf16 [32768, 1024], top-8: 198.7 us, 124.6 us this way.)
+__global__ __launch_bounds__(kThreads) void expand_short_rows_kernel(const uint8_t *x, int64_t row_bytes, const int32_t *token_topk_to_pos,
+                                                                     int num_topk, int kpw, int tpr, int copy_blocks, int num_tokens,
+                                                                     int num_expanded, uint8_t *out, const int32_t *pos_to_expert,
+                                                                     const uint32_t *x_sf, int sf_cols, uint32_t *out_sf,
+                                                                     int64_t out_sf_ld, int sf_col_major, int pad_rows) {
+    const int b = blockIdx.x;
+    if (b < copy_blocks) {
+        // b = 8 * ((token group * groups of positions) + kg) + token within its group of 8
+        const int kgroups = (num_topk + kpw - 1) / kpw;
+        const int q = b >> 3;
+        const int kg = q % kgroups, t = (q / kgroups) * 8 + (b & 7);
+        const int g = (int)threadIdx.x / tpr, i = (int)threadIdx.x - g * tpr;
+        const int k = kg * kpw + g;
+        const int64_t off = (int64_t)i * 16;
+        if (t >= num_tokens || g >= kpw || k >= num_topk) return;
+        const int p = token_topk_to_pos[(int64_t)t * num_topk + k];
+        u32x4 v = u32x4{0u, 0u, 0u, 0u};
+        if (off < row_bytes) v = *reinterpret_cast<const u32x4 *>(x + (int64_t)t * row_bytes + off);   // cached: read num_topk times
+        if (p < 0 || p >= num_expanded) return;
+        if (off < row_bytes) expand_store16(out + (int64_t)p * row_bytes + off, v);
+        if (x_sf)
+            for (int j = i; j < sf_cols; j += tpr)
+                out_sf[sf_col_major ? (int64_t)j * out_sf_ld + p : (int64_t)p * out_sf_ld + j] = x_sf[(int64_t)t * sf_cols + j];
+    } else {
+        expand_zero_padding(b - copy_blocks, pad_rows, num_expanded, row_bytes, out, pos_to_expert, x_sf != nullptr, sf_cols, out_sf, out_sf_ld,
+                            sf_col_major);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // reduce_fused: the inverse of the expansion.  out[t] = sum over k of x[pos(t, k)] * s(t, k), accumulated in fp32 with
 // one fused multiply-add per term, in the order k = 0, 1, ... (so that results are reproducible bit for bit), where
@@ -241,6 +290,35 @@ constexpr int kReduceUnroll = 8;
 template <typename InT> struct ReduceIn;
 template <> struct ReduceIn<bf16_t> { typedef Raw8<bf16_t> raw; };
 template <> struct ReduceIn<float> { typedef Raw8<float> raw; };
+
+// U terms k0 .. k0 + U - 1 of one token: all U rows' pieces are loaded before the first is used
+template <typename InT, int U>
+__device__ __forceinline__ void reduce_terms(float (&acc)[8], const InT *x, const int32_t *pos_row, int k0, int t, int num_topk, int hidden,
+                                             int num_expanded, int col, const float *topk_weights, const float *x_sf) {
+    typename ReduceIn<InT>::raw raw[U];
+    float s[U];
+    bool live[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+        const int k = k0 + j;
+        const int p = uniform_load(pos_row + k);
+        live[j] = p >= 0 && p < num_expanded;
+        // a skipped term reads row 0 (no branch around the loads) and is not added
+        const int row = live[j] ? p : 0;
+        raw[j].load(x + (int64_t)row * hidden + col);
+        s[j] = 1.0f;
+        if (topk_weights) s[j] = live[j] ? uniform_load(topk_weights + (int64_t)t * num_topk + k) : 0.0f;
+        if (x_sf) s[j] = s[j] * uniform_load(x_sf + row);
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+        if (!live[j]) continue;      // wave-uniform
+        float v[8];
+        raw[j].get(v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(v[i], s[j], acc[i]);
+    }
+}
 
 // OUT: 0 bf16, 1 fp32, 2 E4M3
 template <typename InT, int OUT>
@@ -255,31 +333,14 @@ __global__ __launch_bounds__(kThreads) void reduce_fused_kernel(const InT *x, co
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-    for (int k0 = 0; k0 < num_topk; k0 += kReduceUnroll) {
-        typename ReduceIn<InT>::raw raw[kReduceUnroll];
-        float s[kReduceUnroll];
-        bool live[kReduceUnroll];
-#pragma unroll
-        for (int j = 0; j < kReduceUnroll; ++j) {
-            const int k = k0 + j;
-            const int p = k < num_topk ? uniform_load(pos_row + k) : -1;
-            live[j] = p >= 0 && p < num_expanded;
-            // a skipped term reads row 0 (no branch around the loads) and is not added
-            const int row = live[j] ? p : 0;
-            raw[j].load(x + (int64_t)row * hidden + col);
-            s[j] = 1.0f;
-            if (topk_weights) s[j] = live[j] ? uniform_load(topk_weights + (int64_t)t * num_topk + k) : 0.0f;
-            if (x_sf) s[j] = s[j] * uniform_load(x_sf + row);
-        }
-#pragma unroll
-        for (int j = 0; j < kReduceUnroll; ++j) {
-            if (!live[j]) continue;      // wave-uniform
-            float v[8];
-            raw[j].get(v);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(v[i], s[j], acc[i]);
-        }
-    }
+    // whole groups of 8 terms, then the rest in steps of 4, 2 and 1: padding a short list to 8 with skipped terms would
+    // still issue their loads (top-2 of bf16 [8576, 7168]: 46.7 us that way)
+    int k0 = 0;
+    for (; k0 + kReduceUnroll <= num_topk; k0 += kReduceUnroll)
+        reduce_terms<InT, kReduceUnroll>(acc, x, pos_row, k0, t, num_topk, hidden, num_expanded, col, topk_weights, x_sf);
+    if ((num_topk - k0) & 4) { reduce_terms<InT, 4>(acc, x, pos_row, k0, t, num_topk, hidden, num_expanded, col, topk_weights, x_sf); k0 += 4; }
+    if ((num_topk - k0) & 2) { reduce_terms<InT, 2>(acc, x, pos_row, k0, t, num_topk, hidden, num_expanded, col, topk_weights, x_sf); k0 += 2; }
+    if ((num_topk - k0) & 1) reduce_terms<InT, 1>(acc, x, pos_row, k0, t, num_topk, hidden, num_expanded, col, topk_weights, x_sf);
     if (sf) {
         const float f = uniform_load(sf);
 #pragma unroll
@@ -394,16 +455,25 @@ extern "C" int tk_expand_to_fused(const void *x, int64_t num_tokens, int64_t row
                                             x_sf, sf_cols, out_sf, out_sf_ld, sf_col_major);
     if (rc != TK_OK) return rc;
     const int64_t chunks = (row_bytes + kExpandChunk - 1) / kExpandChunk;
-    const int64_t copy_blocks = (num_tokens + 7) / 8 * 8 * num_topk * chunks;
+    // rows of at most half a chunk: several positions of a token per workgroup
+    const int tpr = (int)((row_bytes + 15) / 16);
+    const int kpw = tpr * 2 <= kThreads ? (kThreads / tpr < num_topk ? kThreads / tpr : num_topk) : 1;
+    const int64_t copy_blocks = (num_tokens + 7) / 8 * 8 * (kpw > 1 ? (num_topk + kpw - 1) / kpw : num_topk * chunks);
     // padding workgroups take 8 KB of consecutive rows each, two stores per thread.  Measured (us per call, 1 / 2 / 4
     // rows per workgroup): 8 KB rows 64.4 / 69.7 / 71.0; 4 KB rows with scales 41.4 / 36.0 / 37.0
     const int pad_rows = row_bytes >= 8192 ? 1 : (int)(8192 / row_bytes > 8 ? 8 : 8192 / row_bytes);
     const int64_t grid = copy_blocks + (num_expanded + pad_rows - 1) / pad_rows;
     if (grid == 0) return TK_OK;
-    hipLaunchKernelGGL(expand_to_fused_kernel, dim3((unsigned)grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint8_t *>(x), row_bytes, token_topk_to_pos, num_topk, (int)chunks, (int)copy_blocks,
-                       (int)num_tokens, (int)num_expanded, static_cast<uint8_t *>(out), pos_to_expert,
-                       static_cast<const uint32_t *>(x_sf), sf_cols, static_cast<uint32_t *>(out_sf), out_sf_ld, sf_col_major, pad_rows);
+    if (kpw > 1)
+        hipLaunchKernelGGL(expand_short_rows_kernel, dim3((unsigned)grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const uint8_t *>(x), row_bytes, token_topk_to_pos, num_topk, kpw, tpr, (int)copy_blocks,
+                           (int)num_tokens, (int)num_expanded, static_cast<uint8_t *>(out), pos_to_expert,
+                           static_cast<const uint32_t *>(x_sf), sf_cols, static_cast<uint32_t *>(out_sf), out_sf_ld, sf_col_major, pad_rows);
+    else
+        hipLaunchKernelGGL(expand_to_fused_kernel, dim3((unsigned)grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const uint8_t *>(x), row_bytes, token_topk_to_pos, num_topk, (int)chunks, (int)copy_blocks,
+                           (int)num_tokens, (int)num_expanded, static_cast<uint8_t *>(out), pos_to_expert,
+                           static_cast<const uint32_t *>(x_sf), sf_cols, static_cast<uint32_t *>(out_sf), out_sf_ld, sf_col_major, pad_rows);
     return (int)hipGetLastError();
 }
 
