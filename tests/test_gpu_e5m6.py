@@ -34,7 +34,7 @@ def _inputs(num_tokens, hidden, dtype, seed):
 
 @pytest.mark.parametrize('mode', SF_MODES, ids=lambda m: 'col%d-round%d-packed%d' % tuple(int(v) for v in m))
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32], ids=['bf16', 'f32'])
-@pytest.mark.parametrize('num_tokens,hidden', [(401, 576), (401, 2048), (130, 2560), (67, 7168), (5, 8), (3, 4104), (0, 512)])
+@pytest.mark.parametrize('num_tokens,hidden', [(401, 576), (401, 2048), (130, 2560), (67, 7168), (5, 8), (3, 4104), (0, 512), (9, 11008), (7, 16384), (3, 16392)])
 def test_per_token_cast_to_e5m6(num_tokens, hidden, dtype, mode):
     tk = _tk()
     col, rnd, packed = mode

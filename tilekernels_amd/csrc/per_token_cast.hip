@@ -143,9 +143,9 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
     }
 }
 
-// One scale per row (group == K): a workgroup per row.  Rows of up to ITER * 2048 elements (ITER = 1..4) are held in
-// registers between the amax and the conversion, so they are read once; ITER == 0 takes longer rows in two passes (the
-// second one is served by L2).  Reference: the `hidden == num_per_channels` branch,
+// One scale per row (group == K): a workgroup per row.  Rows of up to 16384 elements are held in registers, ITER pieces
+// of 8 elements per thread, between the amax and the conversion, so they are read once; ITER == 0 takes longer rows
+// in two passes (the second one is served by L2).  Reference: the `hidden == num_per_channels` branch,
 // tile_kernels/quant/per_token_cast_kernel.py:31-35, and the E5M6 cast, which knows no other grouping
 // (per_token_cast_to_e5m6_kernel.py:88).
 template <int FMT> __host__ __device__ constexpr int64_t code_row_bytes(int64_t k) {
@@ -157,6 +157,7 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERN
     TK_PT_KERNEL_UNPACK;
     __shared__ uint32_t part[kThreads / 16];
     const int row = blockIdx.x;
+    const int nt = p.geom;   // threads of the workgroup: 64, 128, 192 or 256, the fewest that cover the row in ITER pieces
     const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row * p.x_ld;   // plain (bf16 / fp32) inputs only
     constexpr int N = ITER > 0 ? ITER : 1;
     Raw8<InT> held[N];
@@ -164,14 +165,16 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERN
     if constexpr (ITER > 0) {
 #pragma unroll
         for (int i = 0; i < ITER; ++i) {
-            const int col = (i * kThreads + threadIdx.x) * 8;
-            held[i].load(x + col, col < p.K);
+            // a lane beyond the end of the row reads the row's first elements (no branch around the loads)
+            const int col = (i * nt + threadIdx.x) * 8;
+            held[i].load(x + (col < p.K ? col : 0));
         }
 #pragma unroll
         for (int i = 0; i < ITER; ++i) {
+            const int col = (i * nt + threadIdx.x) * 8;
             float v[8];
             held[i].get(v);
-            amax = __builtin_fmaxf(amax, absmax8(v));
+            if (col < p.K) amax = __builtin_fmaxf(amax, absmax8(v));
         }
     } else {
         for (int col = threadIdx.x * 8; col < p.K; col += kThreads * 8) {
@@ -187,14 +190,14 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERN
     __syncthreads();
     uint32_t m = 0;
 #pragma unroll
-    for (int i = 0; i < kThreads / 16; ++i) m = umax(m, part[i]);
+    for (int i = 0; i < kThreads / 16; ++i) m = umax(m, i * 16 < nt ? part[i] : 0u);
     const Scale sc = make_scale<Fmt<FMT>::qmax>(u2f(m), Fmt<FMT>::floor_, p.round_sf != 0);
     if (threadIdx.x == 0) sf_store(p.sf, row, 0, sc);
     uint8_t *out_row = p.out + (int64_t)row * code_row_bytes<FMT>(p.K);
     if constexpr (ITER > 0) {
 #pragma unroll
         for (int i = 0; i < ITER; ++i) {
-            const int col = (i * kThreads + threadIdx.x) * 8;
+            const int col = (i * nt + threadIdx.x) * 8;
             float v[8];
             held[i].get(v);
             if (col < p.K) quantise_store8<FMT, false>(v, sc.inv, out_row, col);
@@ -210,16 +213,29 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERN
     }
 }
 
+// Pieces per thread and threads per workgroup of the row kernel: the fewest pieces (of 1, 2, 3, 4, 6, 8) with which at
+// most 256 threads cover the row, then the fewest whole waves that do.  Measured on MI355X, E5M6 cast of bf16, always
+// 256 threads and at most 4 pieces against this: [131072, 512] 86.4 us, [65536, 1536] 67.6 us, [12160, 11008] 89.4 us
+// (two passes).
 template <typename InT, int FMT>
-static void launch_per_token_rowgroup(const PerTokenParams &p, hipStream_t stream) {
-    const int iters = (p.K + kThreads * 8 - 1) / (kThreads * 8);
+static void launch_per_token_rowgroup(PerTokenParams &p, hipStream_t stream) {
+    static const int kPieces[] = {1, 2, 3, 4, 6, 8};
+    int iters = 0, threads = kThreads;
+    for (int it : kPieces) {
+        const int64_t per_wave = (int64_t)it * 64 * 8;
+        const int64_t waves = (p.K + per_wave - 1) / per_wave;
+        if (waves <= kWaves) { iters = it; threads = (int)waves * 64; break; }
+    }
+    p.geom = threads;
 #define TK_ROWGROUP_LAUNCH(I) \
-    hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT, I>), dim3(p.M), dim3(kThreads), 0, stream, TK_PT_LAUNCH_ARGS(p))
+    hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT, I>), dim3(p.M), dim3(threads), 0, stream, TK_PT_LAUNCH_ARGS(p))
     switch (iters) {
         case 1: TK_ROWGROUP_LAUNCH(1); break;
         case 2: TK_ROWGROUP_LAUNCH(2); break;
         case 3: TK_ROWGROUP_LAUNCH(3); break;
         case 4: TK_ROWGROUP_LAUNCH(4); break;
+        case 6: TK_ROWGROUP_LAUNCH(6); break;
+        case 8: TK_ROWGROUP_LAUNCH(8); break;
         default: TK_ROWGROUP_LAUNCH(0); break;
     }
 #undef TK_ROWGROUP_LAUNCH
