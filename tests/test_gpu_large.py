@@ -149,3 +149,37 @@ def test_expand_to_fused_beyond_4_gib():
     want = x[p2t.clamp(min=0).long()]
     want[~live] = 0
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
+def test_more_row_tiles_than_one_grid_plane():
+    """Wide and row-wise tiles put their row tiles on grid.y and grid.z, 32768 per plane: matrices with more row tiles
+    than that (and a last plane that is not full) must give the same result as their halves cast separately, and the
+    oracle's result on windows of rows."""
+    tk = _tk()
+    # per-token cast and its inverse: 2 rows per tile, two column tiles of 7 strips
+    M, K = 2 * 32768 + 2 * 1200 + 1, 7168
+    x = _randn_bf16((M, K), 11)
+    codes, sf = tk.quant.per_token_cast(x, 'e4m3', 128)
+    back = tk.quant.cast_back((codes, sf), 'bf16', (1, 128))
+    h = 32768
+    for a, b in [(0, h), (h, M)]:
+        c2, s2 = tk.quant.per_token_cast(x[a:b], 'e4m3', 128)
+        assert torch.equal(dense_bytes(codes[a:b].cpu()), dense_bytes(c2.cpu())) and torch.equal(sf[a:b], s2)
+        assert torch.equal(back[a:b], tk.quant.cast_back((c2, s2), 'bf16', (1, 128)))
+    for a, b in _windows(M, 9):
+        c_ref, s_ref = torch_ref.cast(x[a:b].cpu(), 'e4m3', (1, 128))
+        _same_bytes(codes[a:b], c_ref, f'codes[{a}:{b}]')
+        _same_bytes(sf[a:b], s_ref, f'sf[{a}:{b}]')
+        _same_bytes(back[a:b], torch_ref.cast_back((c_ref, s_ref), 'bf16', (1, 128)), f'back[{a}:{b}]')
+    del x, codes, sf, back
+    torch.cuda.empty_cache()
+    # SwiGLU cast: 4 rows per tile, two column tiles of 2048 outputs; row-major and packed column-major scales
+    R, H = 4 * 32768 + 4 * 700 + 3, 4096
+    x = _randn_bf16((R, 2 * H), 12)
+    for kw in (dict(), dict(use_tma_aligned_col_major_sf=True, round_sf=True, use_packed_ue8m0=True)):
+        got = tk.quant.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, **kw)
+        for a, b in _windows(R, 8):
+            want = torch_ref.swiglu_forward_and_per_token_cast(x[a:b].cpu(), 'e4m3', 128, **kw)
+            part = tk.quant.swiglu_forward_and_per_token_cast(x[a:b].contiguous(), 'e4m3', 128, **kw)
+            check_fused(part, want, H // 128, bool(kw), f'window [{a}:{b}] alone')
+            assert torch.equal(dense_bytes(got[0][a:b].cpu()), dense_bytes(part[0].cpu())), f'codes[{a}:{b}] {kw}'
