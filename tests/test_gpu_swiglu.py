@@ -87,6 +87,24 @@ def test_swiglu_forward_and_per_token_cast(H, N, with_mask, with_weights, mode, 
     tk.set_num_sms(tk.get_device_num_sms())
 
 
+@pytest.mark.parametrize('mode', [(False, False, False), (True, False, False), (True, True, True)],
+                         ids=lambda m: 'col%d-round%d-packed%d' % tuple(int(v) for v in m))
+@pytest.mark.parametrize('with_mask', [False, True])
+@pytest.mark.parametrize('H', [1024, 2048, 1536, 896, 3584])   # row-wise, wide and stacked tiles of the fp32 kernel (2 pieces per wave)
+def test_swiglu_fp32_input_tiles(H, with_mask, mode):
+    tk = _tk()
+    col, rnd, packed = mode
+    g = torch.Generator().manual_seed(H + int(with_mask))
+    pe, ptt, w = tk.testing.generate_moe_layout(61, 8, 2, 16, g, drop_fraction=0.1)
+    R = pe.numel()
+    x = torch.randn((R, 2 * H), generator=g) * 2
+    x[pe < 0] = 0
+    kw = dict(use_tma_aligned_col_major_sf=col, round_sf=rnd, use_packed_ue8m0=packed)
+    want = torch_ref.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, ptt, w, pe if with_mask else None, **kw)
+    got = tk.quant.swiglu_forward_and_per_token_cast(x.cuda(), 'e4m3', 128, ptt.cuda(), w.cuda(), pe.cuda() if with_mask else None, **kw)
+    check_fused(got, want, H // 128, packed, f'fp32 H={H}')
+
+
 def test_swiglu_fp32_input_and_custom_floor():
     tk = _tk()
     x = torch.randn((50, 512)) * 3

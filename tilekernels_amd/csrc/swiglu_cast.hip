@@ -338,11 +338,13 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KER
 
 // Pieces per wave of the tiled kernel.  Measured on MI355X at [8192, 4096] bf16 (us per call, row-major
 // scales, pieces = rows): 1 row 16.5, 2 rows 15.7, 4 rows 15.0.  With the four pieces taken from one row
-// (T_ROW) instead of four rows (T_WIDE): 14.75 -> 14.63.
+// (T_ROW) instead of four rows (T_WIDE): 14.75 -> 14.63.  fp32 input, whose pieces are twice the bytes (sixteen
+// 16-byte loads per lane with 4 pieces), is better off with 2: [16384, 2 x 2048] 59.5 -> 52.1 us,
+// [16384, 2 x 4096] 116.2 -> 98.2 us.
 #ifndef TK_SWIGLU_RPW
 #define TK_SWIGLU_RPW 4
 #endif
-constexpr int kSwigluRowsPerWave = TK_SWIGLU_RPW;
+template <typename InT> constexpr int swiglu_pieces() { return sizeof(InT) == 4 ? 2 : TK_SWIGLU_RPW; }
 
 template <typename InT, int CLAMP, int RPW, int TILE>
 static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t stream) {
@@ -386,6 +388,7 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
 
 template <typename InT, int CLAMP>
 static hipError_t launch_swiglu_2(SwigluParams &p, bool row_group, int max_blocks, hipStream_t stream) {
+    constexpr int kPieces = swiglu_pieces<InT>();
     if (row_group) {
         const int grid = max_blocks > 0 && max_blocks < p.R ? max_blocks : p.R;
         const int iter = (p.H + kThreads * 8 - 1) / (kThreads * 8);
@@ -399,16 +402,16 @@ static hipError_t launch_swiglu_2(SwigluParams &p, bool row_group, int max_block
             default: TK_ROWGROUP_LAUNCH(0); break;
         }
 #undef TK_ROWGROUP_LAUNCH
-    } else if (p.sf.layout != TK_SF_ROW_F32 && p.H % (kSwigluRowsPerWave * kStripCols) == 0) {
+    } else if (p.sf.layout != TK_SF_ROW_F32 && p.H % (kPieces * kStripCols) == 0) {
         // (other H, where the last column tile of a row is partly empty and the loads are bounds-checked, are
         // better off with stacked tiles: [16384, 2 x 2560] 35.6 us stacked, 44.2 us this way)
-        launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, T_ROWC>(p, max_blocks, stream);
+        launch_swiglu_tiled<InT, CLAMP, kPieces, T_ROWC>(p, max_blocks, stream);
     } else if (p.sf.layout != TK_SF_ROW_F32 || !wide_tiles_pay(p.H)) {
-        launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, T_STACKED>(p, max_blocks, stream);
-    } else if (p.H % (kSwigluRowsPerWave * kStripCols) == 0) {
-        launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, T_ROW>(p, max_blocks, stream);
+        launch_swiglu_tiled<InT, CLAMP, kPieces, T_STACKED>(p, max_blocks, stream);
+    } else if (p.H % (kPieces * kStripCols) == 0) {
+        launch_swiglu_tiled<InT, CLAMP, kPieces, T_ROW>(p, max_blocks, stream);
     } else {
-        launch_swiglu_tiled<InT, CLAMP, kSwigluRowsPerWave, T_WIDE>(p, max_blocks, stream);
+        launch_swiglu_tiled<InT, CLAMP, kPieces, T_WIDE>(p, max_blocks, stream);
     }
     return hipGetLastError();
 }
