@@ -34,7 +34,7 @@ struct SwigluParams {
     unsigned long long *clamped_count;
     int64_t num_weights;
     int R, H;
-    int nwaves, tiles_k;   // waves of a wide tile; tiles along the columns
+    int nwaves, tiles_k;   // waves (= rows) of a T_ROW tile; tiles along the columns
     int round_sf;
     float floor_;        // amax lower clamp
     float clamp;
@@ -89,32 +89,30 @@ __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
 //   T_ROW     (row-major scales, H a multiple of RPW*512): W rows x (RPW*512) columns, one row per wave.  The RPW*4
 //             scales a wave produces are neighbours in the scale row, so the wave stores them itself as one
 //             contiguous run: no LDS stage and no workgroup barrier at the end of the tile
-//   T_WIDE    (row-major scales, other H): RPW rows x (W*512) columns, W waves side by side; the tile's scales are
-//             RPW contiguous runs, staged in LDS and stored as whole segments
 //   T_ROWC    (column-major layouts, H a multiple of RPW*512): the same 4 rows x (RPW*512) columns, one row per wave; the
 //             scales are staged in LDS and stored transposed, 4 rows per run.  Against stacked tiles, whose waves
 //             read 1 KB from each of 8 row halves instead of 4 KB from 2 (us per call, bf16, packed scales):
 //             [32768, 2 x 2048] 60.6 -> 52.4, [16384, 2 x 4096] 69.4 -> 53.9, [8192, 2 x 6144] 48.8 -> 40.9
-//   T_STACKED (other H with column-major layouts, and rows that do not split evenly over the waves of a wide tile): 4*RPW rows x 512 columns, the 4 waves stacked, scales stored
+//   T_STACKED (other H): 4*RPW rows x 512 columns, the 4 waves stacked; the scales are staged in LDS and stored
 //             transposed (row-major: one short run per row)
 // W = blockDim.x / 64.  FULL: the tile grid covers the matrix exactly: no bounds checks are compiled in.
 // MASK: pos_to_expert is given.
-enum { T_STACKED = 0, T_WIDE = 1, T_ROW = 2, T_ROWC = 3 };
+enum { T_STACKED = 0, T_ROW = 2, T_ROWC = 3 };
 
 // ONECOL: the grid is known to be a single column of tiles (else it is found out at run time)
 template <typename InT, int CLAMP, int RPW, int TILE, bool FULL, bool MASK, bool ONECOL>
-__global__ __launch_bounds__(TILE == T_WIDE || TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
+__global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
     TK_SWIGLU_KERNEL_UNPACK;
-    constexpr bool WIDE = TILE == T_WIDE, ROWC = TILE == T_ROWC, ROW = TILE == T_ROW || ROWC;   // ROW: a wave's pieces lie along one row
+    constexpr bool ROWC = TILE == T_ROWC, ROW = TILE == T_ROW || ROWC;   // ROW: a wave's pieces lie along one row
     constexpr bool DIRECT = TILE == T_ROW;  // the wave stores its scales itself
     constexpr int GPS = kStripCols / 128;   // 4 groups per strip
-    constexpr int ROWS = WIDE ? RPW : (ROWC ? kWaves : kWaves * RPW);   // rows per tile (T_ROW: blockDim.x / 64, not used as a constant)
-    constexpr int SGPR = WIDE ? kMaxWideWaves * GPS : (ROWC ? RPW * GPS : GPS);   // staged groups per row (capacity)
+    constexpr int ROWS = ROWC ? kWaves : kWaves * RPW;   // rows per tile (T_ROW: blockDim.x / 64, not used as a constant)
+    constexpr int SGPR = ROWC ? RPW * GPS : GPS;   // staged groups per row
     // The counting variant loops over tiles (its grid is capped so that few workgroups touch the global
     // counters); every other variant has one workgroup per tile on a 2-D grid, which keeps integer
     // divisions and further kernel-argument loads out of the path to the first memory load.
     constexpr bool LOOP = CLAMP == 2;
-    const int nwaves = (WIDE || DIRECT) ? p.nwaves : kWaves;
+    const int nwaves = DIRECT ? p.nwaves : kWaves;
     const int rows = DIRECT ? nwaves : ROWS;
     using RS = RowScales<448, RPW, 16>;
     __shared__ uint32_t stage[DIRECT ? 1 : ROWS][DIRECT ? 1 : SGPR];
@@ -123,14 +121,14 @@ __global__ __launch_bounds__(TILE == T_WIDE || TILE == T_ROW ? 64 * kMaxWideWave
     const int lane = threadIdx.x & 63, wave = wave_id();
     const bool has_weight = p.pos_to_token_topk != nullptr;
     const int own = lane & 15;
-    const int srow = WIDE ? 0 : (ROWC ? wave : wave * RPW);
+    const int srow = ROWC ? wave : wave * RPW;
     ClampCounter<CLAMP> counter;
 
     for (int tile = LOOP ? (int)blockIdx.x : 0; tile < total; tile += LOOP ? (int)gridDim.x : 1) {
         const int tile_m = LOOP ? tile / p.tiles_k : tile_grid_row(ONECOL || p.tiles_k == 1);
         const int tile_k = LOOP ? tile - tile_m * p.tiles_k : tile_grid_col(ONECOL || p.tiles_k == 1);
         // piece r of the wave: row `row0 + (ROW ? 0 : r)`, columns from `col + (ROW ? r * 512 : 0)`
-        const int strip = ROW ? tile_k * RPW : (WIDE ? tile_k * nwaves + wave : tile_k);
+        const int strip = ROW ? tile_k * RPW : tile_k;
         const int col = strip * kStripCols + lane * 8;
         const int row0 = ROW ? tile_m * nwaves + wave : tile_m * ROWS + srow;
         const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * (2 * (int64_t)p.H) + col;
@@ -220,7 +218,7 @@ __global__ __launch_bounds__(TILE == T_WIDE || TILE == T_ROW ? 64 * kMaxWideWave
                     if (FULL || (row0 < p.R && k < p.sf.nk))
                         st_stream4(reinterpret_cast<float *>(p.sf.base) + (int64_t)row0 * p.sf.ld + k, f2u(rs.own[c].sf));
                 } else {
-                    stage[srow + c * RS::A + own][(WIDE ? wave * GPS : 0) + (lane >> 4)] =
+                    stage[srow + c * RS::A + own][lane >> 4] =
                         p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
                 }
             }
@@ -233,7 +231,6 @@ __global__ __launch_bounds__(TILE == T_WIDE || TILE == T_ROW ? 64 * kMaxWideWave
         if constexpr (!DIRECT) {
             __syncthreads();
             if (ROWC) sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
-            else if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
             else if (p.sf.layout == TK_SF_ROW_F32) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, GPS, tile_m * ROWS, tile_k * GPS);
             else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
             if (LOOP && (int)gridDim.x < total) __syncthreads();   // stage is reused by the next tile
@@ -338,7 +335,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KER
 
 // Pieces per wave of the tiled kernel.  Measured on MI355X at [8192, 4096] bf16 (us per call, row-major
 // scales, pieces = rows): 1 row 16.5, 2 rows 15.7, 4 rows 15.0.  With the four pieces taken from one row
-// (T_ROW) instead of four rows (T_WIDE): 14.75 -> 14.63.  fp32 input, whose pieces are twice the bytes (sixteen
+// (T_ROW) instead of four rows: 14.75 -> 14.63.  fp32 input, whose pieces are twice the bytes (sixteen
 // 16-byte loads per lane with 4 pieces), is better off with 2: [16384, 2 x 2048] 59.5 -> 52.1 us,
 // [16384, 2 x 4096] 116.2 -> 98.2 us.
 #ifndef TK_SWIGLU_RPW
@@ -352,9 +349,9 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
     // T_ROW, rows per workgroup (= waves), us per call at [8192, 4096] dense / [48128, 4096] with a third of the rows
     // masked: 1: 14.9 / 61.6, 2: 14.85 / 62.1, 4: 14.68 / 62.9, 8: 15.15 / 63.4.  A masked batch is better off with
     // single-wave workgroups: a wave whose row is padding is done at once and frees its slot alone.
-    const int waves = TILE == T_WIDE ? wide_tile_waves(strips) : (TILE == T_ROW && p.pos_to_expert ? 1 : kWaves);
-    const int rows = TILE == T_WIDE ? RPW : (TILE == T_ROW || TILE == T_ROWC ? waves : kWaves * RPW);
-    const int cols = TILE == T_WIDE ? waves * kStripCols : (TILE == T_ROW || TILE == T_ROWC ? RPW * kStripCols : kStripCols);
+    const int waves = TILE == T_ROW && p.pos_to_expert ? 1 : kWaves;
+    const int rows = TILE == T_ROW || TILE == T_ROWC ? waves : kWaves * RPW;
+    const int cols = TILE == T_ROW || TILE == T_ROWC ? RPW * kStripCols : kStripCols;
     const int tiles_m = (p.R + rows - 1) / rows;
     p.tiles_k = (p.H + cols - 1) / cols;
     p.nwaves = waves;
@@ -406,12 +403,12 @@ static hipError_t launch_swiglu_2(SwigluParams &p, bool row_group, int max_block
         // (other H, where the last column tile of a row is partly empty and the loads are bounds-checked, are
         // better off with stacked tiles: [16384, 2 x 2560] 35.6 us stacked, 44.2 us this way)
         launch_swiglu_tiled<InT, CLAMP, kPieces, T_ROWC>(p, max_blocks, stream);
-    } else if (p.sf.layout != TK_SF_ROW_F32 || !wide_tiles_pay(p.H)) {
-        launch_swiglu_tiled<InT, CLAMP, kPieces, T_STACKED>(p, max_blocks, stream);
     } else if (p.H % (kPieces * kStripCols) == 0) {
         launch_swiglu_tiled<InT, CLAMP, kPieces, T_ROW>(p, max_blocks, stream);
     } else {
-        launch_swiglu_tiled<InT, CLAMP, kPieces, T_WIDE>(p, max_blocks, stream);
+        // (tiles of a few rows with the workgroup's waves side by side, as the per-token cast uses them for row-major
+        // scales, are no faster here: bf16 [26112, 2 x 2560] 52.9 us against 51.2 us, [21760, 2 x 3072] 53.1 against 51.5)
+        launch_swiglu_tiled<InT, CLAMP, kPieces, T_STACKED>(p, max_blocks, stream);
     }
     return hipGetLastError();
 }
