@@ -44,41 +44,51 @@ struct PerTokenParams {
     (p).x, (p).x_ld, (p).xsf.base, (p).xsf.ld, (p).M, (p).K, (p).geom, (p).xsf.layout, (p).in_bm, (p).in_bk, (p).out, \
         (p).sf.base, (p).sf.ld, (p).round_sf, (p).mode, (p).sf.layout, (p).sf.nk, (p).xsf.nm, (p).xsf.nk
 
-// Tile shapes (RPW = rows per wave):
-//   WIDE  (row-major scales):      RPW rows x (W*512) columns, W = blockDim.x/64 waves side by side on the same rows;
-//         the tile's scales are RPW contiguous runs, staged in LDS and stored as whole segments
-//   !WIDE (column-major layouts, and rows of at most 1024 columns):  4*RPW rows x 512 columns, the 4 waves stacked;
-//         the staged scales are stored transposed, 4*RPW rows per contiguous segment (row-major: one short run per row)
+// Tile shapes (RPW = pieces of 8 elements per lane, i.e. of 512 columns per wave):
+//   T_WIDE    (row-major scales):      RPW rows x (W*512) columns, W = blockDim.x/64 waves side by side on the same rows;
+//             the tile's scales are RPW contiguous runs, staged in LDS and stored as whole segments
+//   T_STACKED (column-major layouts, and rows of at most 1024 columns):  4*RPW rows x 512 columns, the 4 waves stacked;
+//             the staged scales are stored transposed, 4*RPW rows per contiguous segment (row-major: one short run per row)
+//   T_ROWWISE (row-major scales, K a multiple of RPW*512, whole tiles only): 4 rows x (RPW*512) columns, one row per
+//             wave; the scales a wave produces are neighbours in the scale row and it stores them itself: no LDS
+//             stage and no barrier
 // FULL: the tile grid covers the matrix exactly, so no bounds checks are compiled in.
-template <typename InT, int G, int FMT, int RPW, bool WIDE, bool FULL>
-__global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_token_cast_kernel(TK_PT_KERNEL_ARGS) {
+enum { T_STACKED = 0, T_WIDE = 1, T_ROWWISE = 2 };
+
+template <typename InT, int G, int FMT, int RPW, int TILE, bool FULL>
+__global__ __launch_bounds__(TILE == T_WIDE ? 64 * kMaxWideWaves : kThreads) void per_token_cast_kernel(TK_PT_KERNEL_ARGS) {
     TK_PT_KERNEL_UNPACK;
+    constexpr bool WIDE = TILE == T_WIDE, ROWW = TILE == T_ROWWISE;
+    static_assert(!ROWW || FULL, "row-wise tiles are launched on whole tiles only");
     constexpr int LPG = G / 8;            // lanes per group
     constexpr int GPS = kStripCols / G;   // groups per 512-column strip
-    constexpr int ROWS = WIDE ? RPW : kWaves * RPW;       // rows per tile
+    constexpr int ROWS = WIDE ? RPW : kWaves * RPW;       // rows per tile (stacked and wide)
     constexpr int SGPR = WIDE ? kMaxWideWaves * GPS : GPS;   // staged groups per row (capacity)
     // everything on the way to the first load comes from the preloaded arguments and the workgroup ids
     const int nwaves = WIDE ? p.geom : kWaves;
     using RS = RowScales<Fmt<FMT>::qmax, RPW, LPG>;
-    __shared__ uint32_t stage[ROWS][SGPR];
+    __shared__ uint32_t stage[ROWW ? 1 : ROWS][ROWW ? 1 : SGPR];
 
-    const bool one_col = p.geom * kStripCols >= p.K;   // wide tiles: the waves of one tile cover a whole row
-    const int tile_m = WIDE ? tile_grid_row(one_col) : (int)blockIdx.x / p.geom;
-    const int tile_k = WIDE ? tile_grid_col(one_col) : (int)blockIdx.x - tile_m * p.geom;
+    // wide tiles: the waves of one tile cover a whole row; row-wise: one wave does
+    const bool one_col = (ROWW ? RPW : p.geom) * kStripCols >= p.K;
+    const int tile_m = (WIDE || ROWW) ? tile_grid_row(one_col) : (int)blockIdx.x / p.geom;
+    const int tile_k = (WIDE || ROWW) ? tile_grid_col(one_col) : (int)blockIdx.x - tile_m * p.geom;
     const int lane = threadIdx.x & 63, wave = wave_id();
-    const int strip = WIDE ? tile_k * nwaves + wave : tile_k;
+    // piece r of the wave: row `row0 + (ROWW ? 0 : r)`, columns from `col + (ROWW ? r * 512 : 0)`
+    const int strip = WIDE ? tile_k * nwaves + wave : (ROWW ? tile_k * RPW : tile_k);
     const int col = strip * kStripCols + lane * 8;
     const int g_in_strip = lane / LPG;
     const int kgrp = strip * GPS + g_in_strip;
     const bool col_ok = FULL || col < p.K;
     const int srow = WIDE ? 0 : wave * RPW;                // first staged row of this wave
-    const int row0 = tile_m * ROWS + srow;
+    const int row0 = ROWW ? tile_m * kWaves + wave : tile_m * ROWS + srow;
     const int64_t out_ld = FMT == TK_E4M3 ? p.K : p.K / 2;
+    constexpr int kRowStep = ROWW ? 0 : 1, kColStep = ROWW ? kStripCols : 0, kGrpStep = ROWW ? GPS : 0;
 
     Raw8<InT> raw[RPW];
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
-        const void *xp = elem_ptr<InT>(p.x, row0 + r, p.x_ld, col);
+        const void *xp = elem_ptr<InT>(p.x, row0 + r * kRowStep, p.x_ld, col + r * kColStep);
         if (FULL) {
             raw[r].load(xp);
         } else {
@@ -91,7 +101,7 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
         if constexpr (Elem<InT>::quantised) {
             // the 8 codes of a lane share one input scale (input blocks are at least 32 columns wide)
             const bool ok = col_ok && (FULL || row0 + r < p.M);
-            raw[r].s = ok ? sf_load(p.xsf, (row0 + r) / p.in_bm, col / p.in_bk) : 0.0f;
+            raw[r].s = ok ? sf_load(p.xsf, (row0 + r * kRowStep) / p.in_bm, (col + r * kColStep) / p.in_bk) : 0.0f;
         }
     }
 
@@ -100,7 +110,7 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
             const bool ok = col_ok && (FULL || row0 + r < p.M);
-            inv[r] = 1.0f / (ok ? sf_load_select(p.sf, row0 + r, kgrp) : 1.0f);
+            inv[r] = 1.0f / (ok ? sf_load_select(p.sf, row0 + r * kRowStep, kgrp + r * kGrpStep) : 1.0f);
         }
     } else {
         float amax[RPW];
@@ -114,13 +124,19 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
         rs.compute(amax, Fmt<FMT>::floor_, p.round_sf != 0, lane);
 #pragma unroll
         for (int r = 0; r < RPW; ++r) inv[r] = rs.inv[r];
-        // lane j (< A) of a group computed the scale of row c*A + j
+        // lane j (< A) of a group computed the scale of piece c*A + j
         const int own = lane % LPG;
         if (own < RS::A) {
 #pragma unroll
-            for (int c = 0; c < RS::NC; ++c)
-                stage[srow + c * RS::A + own][(WIDE ? wave * GPS : 0) + g_in_strip] =
-                    p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
+            for (int c = 0; c < RS::NC; ++c) {
+                if constexpr (ROWW) {
+                    // group g_in_strip of piece c*A + own: the wave's scales form one run of RPW * GPS floats
+                    st_stream4(reinterpret_cast<float *>(p.sf.base) + (int64_t)row0 * p.sf.ld + kgrp + (c * RS::A + own) * GPS, f2u(rs.own[c].sf));
+                } else {
+                    stage[srow + c * RS::A + own][(WIDE ? wave * GPS : 0) + g_in_strip] =
+                        p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
+                }
+            }
         }
     }
     if (p.mode != TK_SF_ONLY) {
@@ -129,17 +145,19 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void per_toke
             if (col_ok && (FULL || row0 + r < p.M)) {
                 float v[8];
                 raw[r].get(v);
-                uint8_t *out_row = p.out + (int64_t)(row0 + r) * out_ld;
-                if (p.mode == TK_CAST_GIVEN_SF) quantise_store8<FMT, true>(v, inv[r], out_row, col);
-                else quantise_store8<FMT, false>(v, inv[r], out_row, col);
+                uint8_t *out_row = p.out + (int64_t)(row0 + r * kRowStep) * out_ld;
+                if (p.mode == TK_CAST_GIVEN_SF) quantise_store8<FMT, true>(v, inv[r], out_row, col + r * kColStep);
+                else quantise_store8<FMT, false>(v, inv[r], out_row, col + r * kColStep);
             }
         }
     }
-    if (p.mode != TK_CAST_GIVEN_SF) {
-        __syncthreads();
-        if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
-        else if (p.sf.layout == TK_SF_ROW_F32) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, GPS, tile_m * ROWS, tile_k * GPS);
-        else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
+    if constexpr (!ROWW) {
+        if (p.mode != TK_CAST_GIVEN_SF) {
+            __syncthreads();
+            if (WIDE) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, nwaves * GPS, tile_m * ROWS, tile_k * nwaves * GPS);
+            else if (p.sf.layout == TK_SF_ROW_F32) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, GPS, tile_m * ROWS, tile_k * GPS);
+            else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
+        }
     }
 }
 
@@ -247,28 +265,41 @@ static void launch_per_token_rowgroup(PerTokenParams &p, hipStream_t stream) {
 // its fixed work; E4M3 1x128 [8192, 4096] -> E2M1 1x32: 14.3 / 12.0 / 12.2 for 2 / 4 / 8 rows.
 template <typename InT> constexpr int rows_per_wave() { return Elem<InT>::quantised ? 4 : 2; }
 
-template <typename InT, int G, int FMT, bool WIDE>
+template <typename InT, int G, int FMT, int TILE>
 static void launch_per_token_tiled(PerTokenParams &p, hipStream_t stream) {
     constexpr int RPW = rows_per_wave<InT>();
+    constexpr bool WIDE = TILE == T_WIDE, ROWW = TILE == T_ROWWISE;
     const int strips = (p.K + kStripCols - 1) / kStripCols;
     const int waves = WIDE ? wide_tile_waves(strips) : kWaves;
-    const int rows = WIDE ? RPW : kWaves * RPW;
-    const int cols = WIDE ? waves * kStripCols : kStripCols;
+    const int rows = WIDE ? RPW : (ROWW ? kWaves : kWaves * RPW);
+    const int cols = WIDE ? waves * kStripCols : (ROWW ? RPW * kStripCols : kStripCols);
     const int tiles_m = (p.M + rows - 1) / rows, tiles_k = (p.K + cols - 1) / cols;
     p.geom = WIDE ? waves : tiles_k;
     const dim3 block(64 * waves);
-    const dim3 grid = WIDE ? tile_grid(tiles_k, tiles_m) : dim3((unsigned)(tiles_m * tiles_k));
-    if (p.M % rows == 0 && p.K % cols == 0 && (!WIDE || tile_grid_exact(tiles_k, tiles_m)))
-        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, true>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
-    else
-        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, WIDE, false>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
+    const dim3 grid = (WIDE || ROWW) ? tile_grid(tiles_k, tiles_m) : dim3((unsigned)(tiles_m * tiles_k));
+    if constexpr (ROWW) {
+        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, TILE, true>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
+    } else {
+        if (p.M % rows == 0 && p.K % cols == 0 && (!WIDE || tile_grid_exact(tiles_k, tiles_m)))
+            hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, TILE, true>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
+        else
+            hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, TILE, false>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
+    }
 }
 
 template <typename InT, int G, int FMT>
 static void launch_per_token_group(PerTokenParams &p, hipStream_t stream) {
+    constexpr int RPW = rows_per_wave<InT>();
+    const int tiles_m = (p.M + kWaves - 1) / kWaves, tiles_k = p.K / (RPW * kStripCols);
+    // Row-wise tiles where they fit exactly.  Measured on MI355X against wide tiles: bf16 [4096, 7168] -> E4M3 14.85 ->
+    // 14.46 us, [32768, 4096] 59.4 -> 56.8 us, given scales 15.83 -> 15.61 us; the scale-only mode, whose only stores
+    // are the scales, is better off with the staged runs of the wide tile (10.15 us against 10.85 us).
+    if (p.sf.layout == TK_SF_ROW_F32 && p.mode != TK_SF_ONLY && p.K % (RPW * kStripCols) == 0 && p.M % kWaves == 0 &&
+        tile_grid_exact(tiles_k, tiles_m))
+        launch_per_token_tiled<InT, G, FMT, T_ROWWISE>(p, stream);
     // a caller-supplied scale tensor is only read, so either tile shape does
-    if (p.sf.layout == TK_SF_ROW_F32 && wide_tiles_pay(p.K)) launch_per_token_tiled<InT, G, FMT, true>(p, stream);
-    else launch_per_token_tiled<InT, G, FMT, false>(p, stream);
+    else if (p.sf.layout == TK_SF_ROW_F32 && wide_tiles_pay(p.K)) launch_per_token_tiled<InT, G, FMT, T_WIDE>(p, stream);
+    else launch_per_token_tiled<InT, G, FMT, T_STACKED>(p, stream);
 }
 
 // plain (bf16 / fp32) and quantised (codes + block scales) inputs alike; one scale per row (group == K
