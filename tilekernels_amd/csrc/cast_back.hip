@@ -118,6 +118,8 @@ static void launch_cast_back_2(const void *x, void *out, const void *sf, int64_t
 template <typename InT, bool OUT_F32>
 static hipError_t launch_cast_back(const void *x, void *out, const void *sf, int64_t sf_ld, int M, int K, int sf_layout,
                                    int bm, int bk, hipStream_t stream) {
+    // (one row per wave with its pieces along the row, the shape that pays in the per-token cast, measured within 2 % here
+    // either way: E4M3 [8192, 4096] to bf16 17.25 -> 17.43 us, to fp32 29.63 -> 29.08 us)
     // wide tiles with column-major scales are no faster (E4M3 [8192, 4096]) and slower with 32 x 32 blocks (20.9 us
     // against 16.2 us): a 2-row tile then uses 8 bytes of each scale line it touches
     if (sf_layout == TK_SF_ROW_F32 && wide_tiles_pay(K)) launch_cast_back_2<InT, OUT_F32, true>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);
