@@ -170,12 +170,15 @@ template <int FMT> __host__ __device__ constexpr int64_t code_row_bytes(int64_t 
     return FMT == TK_E4M3 ? k : (FMT == TK_E2M1 ? k / 2 : k / 8 * 12);
 }
 
-template <typename InT, int FMT, int ITER>
+// NT: threads of the workgroup when known at compile time (256), else 0: the count is read from the arguments.
+// EXACT: the row is exactly ITER * NT * 8 elements long, no bounds checks.  (Both for the common row lengths: the
+// E5M6 cast of bf16 [8192, 4096] measures 20.4 us without them, 20.1 us with NT alone.)
+template <typename InT, int FMT, int ITER, int NT, bool EXACT>
 __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERNEL_ARGS) {
     TK_PT_KERNEL_UNPACK;
     __shared__ uint32_t part[kThreads / 16];
     const int row = blockIdx.x;
-    const int nt = p.geom;   // threads of the workgroup: 64, 128, 192 or 256, the fewest that cover the row in ITER pieces
+    const int nt = NT ? NT : p.geom;   // threads of the workgroup: 64, 128, 192 or 256, the fewest that cover the row in ITER pieces
     const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row * p.x_ld;   // plain (bf16 / fp32) inputs only
     constexpr int N = ITER > 0 ? ITER : 1;
     Raw8<InT> held[N];
@@ -185,14 +188,14 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERN
         for (int i = 0; i < ITER; ++i) {
             // a lane beyond the end of the row reads the row's first elements (no branch around the loads)
             const int col = (i * nt + threadIdx.x) * 8;
-            held[i].load(x + (col < p.K ? col : 0));
+            held[i].load(x + ((EXACT || col < p.K) ? col : 0));
         }
 #pragma unroll
         for (int i = 0; i < ITER; ++i) {
             const int col = (i * nt + threadIdx.x) * 8;
             float v[8];
             held[i].get(v);
-            if (col < p.K) amax = __builtin_fmaxf(amax, absmax8(v));
+            if (EXACT || col < p.K) amax = __builtin_fmaxf(amax, absmax8(v));
         }
     } else {
         for (int col = threadIdx.x * 8; col < p.K; col += kThreads * 8) {
@@ -218,7 +221,7 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERN
             const int col = (i * nt + threadIdx.x) * 8;
             float v[8];
             held[i].get(v);
-            if (col < p.K) quantise_store8<FMT, false>(v, sc.inv, out_row, col);
+            if (EXACT || col < p.K) quantise_store8<FMT, false>(v, sc.inv, out_row, col);
         }
     } else {
         for (int col = threadIdx.x * 8; col < p.K; col += kThreads * 8) {
@@ -245,8 +248,15 @@ static void launch_per_token_rowgroup(PerTokenParams &p, hipStream_t stream) {
         if (waves <= kWaves) { iters = it; threads = (int)waves * 64; break; }
     }
     p.geom = threads;
-#define TK_ROWGROUP_LAUNCH(I) \
-    hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT, I>), dim3(p.M), dim3(threads), 0, stream, TK_PT_LAUNCH_ARGS(p))
+#define TK_ROWGROUP_LAUNCH(I)                                                                                                             \
+    do {                                                                                                                                  \
+        if (threads == kThreads && p.K == (I) * kThreads * 8)                                                                             \
+            hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT, I, kThreads, (I) != 0>), dim3(p.M), dim3(threads), 0, stream, TK_PT_LAUNCH_ARGS(p)); \
+        else if (threads == kThreads)                                                                                                     \
+            hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT, I, kThreads, false>), dim3(p.M), dim3(threads), 0, stream, TK_PT_LAUNCH_ARGS(p)); \
+        else                                                                                                                              \
+            hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT, I, 0, false>), dim3(p.M), dim3(threads), 0, stream, TK_PT_LAUNCH_ARGS(p));   \
+    } while (0)
     switch (iters) {
         case 1: TK_ROWGROUP_LAUNCH(1); break;
         case 2: TK_ROWGROUP_LAUNCH(2); break;
