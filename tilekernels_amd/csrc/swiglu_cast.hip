@@ -18,10 +18,6 @@
 #define TK_TRACE(point)
 #endif
 
-#ifndef TK_MASK_BRANCHLESS
-#define TK_MASK_BRANCHLESS 1
-#endif
-
 namespace tk {
 
 struct SwigluParams {
@@ -153,7 +149,7 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
             if (FULL && !MASK) {
                 rg[r].load(xr);
                 ru[r].load(xr + p.H);
-            } else if (TK_MASK_BRANCHLESS) {
+            } else {
                 // no branch around the loads (a branch would make the compiler wait for all eight loads
                 // before the first row is evaluated): a padding row, and a lane beyond the last row or column,
                 // reads the first bytes of the matrix, which every wave shares, and is cleared by value
@@ -162,9 +158,6 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
                 rg[r].load(src);
                 ru[r].load(ok ? xr + p.H : src);
                 if (!ok) { rg[r].zero(); ru[r].zero(); }
-            } else {
-                rg[r].load(xr, live[r] && piece_ok);
-                ru[r].load(xr + p.H, live[r] && piece_ok);
             }
         }
 
