@@ -338,7 +338,6 @@ template <typename InT> constexpr int swiglu_pieces() { return sizeof(InT) == 4 
 
 template <typename InT, int CLAMP, int RPW, int TILE>
 static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t stream) {
-    const int strips = (p.H + kStripCols - 1) / kStripCols;
     // T_ROW, rows per workgroup (= waves), us per call at [8192, 4096] dense / [48128, 4096] with a third of the rows
     // masked: 1: 14.9 / 61.6, 2: 14.85 / 62.1, 4: 14.68 / 62.9, 8: 15.15 / 63.4.  A masked batch is better off with
     // single-wave workgroups: a wave whose row is padding is done at once and frees its slot alone.
