@@ -242,13 +242,14 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KER
     TK_SWIGLU_KERNEL_UNPACK;
     __shared__ uint32_t part[kThreads / 16];
     const InT *xb = reinterpret_cast<const InT *>(p.x);
+    const int nt = p.nwaves * 64;   // threads of the workgroup: the fewest whole waves that cover a row in ITER pieces
     ClampCounter<CLAMP> counter;
     for (int row = blockIdx.x; row < p.R; row += gridDim.x) {
         const bool live = p.pos_to_expert == nullptr || p.pos_to_expert[row] >= 0;
         uint8_t *out_row = p.out + (int64_t)row * p.H;
         float *sf_row = reinterpret_cast<float *>(p.sf.base) + (int64_t)row * p.sf.ld;
         if (!live) {
-            for (int col = threadIdx.x * 8; col < p.H; col += kThreads * 8) st_stream8(out_row + col, u32x2{0u, 0u});
+            for (int col = threadIdx.x * 8; col < p.H; col += nt * 8) st_stream8(out_row + col, u32x2{0u, 0u});
             if (threadIdx.x == 0) sf_row[0] = 0.0f;
             continue;
         }
@@ -262,14 +263,14 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KER
 #pragma unroll
             for (int i = 0; i < ITER; ++i) {
                 // a lane beyond the end of the row reads the row's first elements (no branch around the loads)
-                const int col = (i * kThreads + threadIdx.x) * 8;
+                const int col = (i * nt + threadIdx.x) * 8;
                 const int c = col < p.H ? col : 0;
                 rg[i].load(x + c);
                 ru[i].load(x + p.H + c);
             }
 #pragma unroll
             for (int i = 0; i < ITER; ++i) {
-                const int col = (i * kThreads + threadIdx.x) * 8;
+                const int col = (i * nt + threadIdx.x) * 8;
                 float g[8], u[8];
                 rg[i].get(g);
                 ru[i].get(u);
@@ -291,20 +292,20 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KER
                 __syncthreads();
                 uint32_t m = 0;
 #pragma unroll
-                for (int i = 0; i < kThreads / 16; ++i) m = umax(m, part[i]);
+                for (int i = 0; i < kThreads / 16; ++i) m = umax(m, i * 16 < nt ? part[i] : 0u);
                 const Scale sc = make_scale<448>(u2f(m), p.floor_, p.round_sf != 0);
                 inv = sc.inv;
                 if (threadIdx.x == 0) sf_row[0] = sc.sf;
                 if constexpr (ITER > 0) {
 #pragma unroll
                     for (int i = 0; i < ITER; ++i) {
-                        const int col = (i * kThreads + threadIdx.x) * 8;
+                        const int col = (i * nt + threadIdx.x) * 8;
                         if (col < p.H) quantise_store8<TK_E4M3, false>(held[i], inv, out_row, col);
                     }
                     continue;
                 }
             }
-            for (int col = threadIdx.x * 8; col < p.H; col += kThreads * 8) {
+            for (int col = threadIdx.x * 8; col < p.H; col += nt * 8) {
                 Raw8<InT> rg, ru;
                 rg.load_cached(x + col);
                 ru.load_cached(x + p.H + col);
@@ -380,10 +381,17 @@ static hipError_t launch_swiglu_2(SwigluParams &p, bool row_group, int max_block
     constexpr int kPieces = swiglu_pieces<InT>();
     if (row_group) {
         const int grid = max_blocks > 0 && max_blocks < p.R ? max_blocks : p.R;
-        const int iter = (p.H + kThreads * 8 - 1) / (kThreads * 8);
+        // the fewest pieces per thread (1..4) with which at most 4 waves cover a row, then the fewest waves that do
+        // (bf16 [65536, 2 x 512]: 65 us with 256 threads per row whatever its length)
+        int iter = 0, waves = kWaves;
+        for (int it = 1; it <= 4 && iter == 0; ++it) {
+            const int w = (p.H + it * kStripCols - 1) / (it * kStripCols);
+            if (w <= kWaves) { iter = it; waves = w; }
+        }
+        p.nwaves = waves;
 #define TK_ROWGROUP_LAUNCH(ITER) \
-    hipLaunchKernelGGL((swiglu_rowgroup_kernel<InT, CLAMP, ITER>), dim3(grid), dim3(kThreads), 0, stream, TK_SWIGLU_LAUNCH_ARGS(p))
-        switch (iter <= 4 ? iter : 0) {
+    hipLaunchKernelGGL((swiglu_rowgroup_kernel<InT, CLAMP, ITER>), dim3(grid), dim3(64 * waves), 0, stream, TK_SWIGLU_LAUNCH_ARGS(p))
+        switch (iter) {
             case 1: TK_ROWGROUP_LAUNCH(1); break;
             case 2: TK_ROWGROUP_LAUNCH(2); break;
             case 3: TK_ROWGROUP_LAUNCH(3); break;
