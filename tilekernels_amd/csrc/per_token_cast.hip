@@ -49,17 +49,19 @@ struct PerTokenParams {
 //             the tile's scales are RPW contiguous runs, staged in LDS and stored as whole segments
 //   T_STACKED (column-major layouts, and rows of at most 1024 columns):  4*RPW rows x 512 columns, the 4 waves stacked;
 //             the staged scales are stored transposed, 4*RPW rows per contiguous segment (row-major: one short run per row)
-//   T_ROWWISE (row-major scales, K a multiple of RPW*512, whole tiles only): 4 rows x (RPW*512) columns, one row per
+//   T_ROWWISE (row-major scales, K a multiple of RPW*512): 4 rows x (RPW*512) columns, one row per
 //             wave; the scales a wave produces are neighbours in the scale row and it stores them itself: no LDS
 //             stage and no barrier
-// FULL: the tile grid covers the matrix exactly, so no bounds checks are compiled in.
+// FULL_GRID: the tile grid covers the matrix exactly, so no bounds checks are compiled in.
 enum { T_STACKED = 0, T_WIDE = 1, T_ROWWISE = 2 };
 
-template <typename InT, int G, int FMT, int RPW, int TILE, bool FULL>
+template <typename InT, int G, int FMT, int RPW, int TILE, bool FULL_GRID>
 __global__ __launch_bounds__(TILE == T_WIDE ? 64 * kMaxWideWaves : kThreads) void per_token_cast_kernel(TK_PT_KERNEL_ARGS) {
     TK_PT_KERNEL_UNPACK;
     constexpr bool WIDE = TILE == T_WIDE, ROWW = TILE == T_ROWWISE;
-    static_assert(!ROWW || FULL, "row-wise tiles are launched on whole tiles only");
+    // row-wise tiles always fit the columns, and their waves share nothing: on a grid that overhangs the last row the
+    // waves beyond it leave at once and the others run without bounds checks, like on an exact grid
+    constexpr bool FULL = FULL_GRID || ROWW;
     constexpr int LPG = G / 8;            // lanes per group
     constexpr int GPS = kStripCols / G;   // groups per 512-column strip
     constexpr int ROWS = WIDE ? RPW : kWaves * RPW;       // rows per tile (stacked and wide)
@@ -82,6 +84,9 @@ __global__ __launch_bounds__(TILE == T_WIDE ? 64 * kMaxWideWaves : kThreads) voi
     const bool col_ok = FULL || col < p.K;
     const int srow = WIDE ? 0 : wave * RPW;                // first staged row of this wave
     const int row0 = ROWW ? tile_m * kWaves + wave : tile_m * ROWS + srow;
+    if constexpr (ROWW && !FULL_GRID) {
+        if (row0 >= p.M) return;
+    }
     const int64_t out_ld = FMT == TK_E4M3 ? p.K : p.K / 2;
     constexpr int kRowStep = ROWW ? 0 : 1, kColStep = ROWW ? kStripCols : 0, kGrpStep = ROWW ? GPS : 0;
 
@@ -287,25 +292,19 @@ static void launch_per_token_tiled(PerTokenParams &p, hipStream_t stream) {
     p.geom = WIDE ? waves : tiles_k;
     const dim3 block(64 * waves);
     const dim3 grid = (WIDE || ROWW) ? tile_grid(tiles_k, tiles_m) : dim3((unsigned)(tiles_m * tiles_k));
-    if constexpr (ROWW) {
+    if (p.M % rows == 0 && p.K % cols == 0 && (!(WIDE || ROWW) || tile_grid_exact(tiles_k, tiles_m)))
         hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, TILE, true>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
-    } else {
-        if (p.M % rows == 0 && p.K % cols == 0 && (!WIDE || tile_grid_exact(tiles_k, tiles_m)))
-            hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, TILE, true>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
-        else
-            hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, TILE, false>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
-    }
+    else
+        hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, TILE, false>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
 }
 
 template <typename InT, int G, int FMT>
 static void launch_per_token_group(PerTokenParams &p, hipStream_t stream) {
     constexpr int RPW = rows_per_wave<InT>();
-    const int tiles_m = (p.M + kWaves - 1) / kWaves, tiles_k = p.K / (RPW * kStripCols);
-    // Row-wise tiles where they fit exactly.  Measured on MI355X against wide tiles: bf16 [4096, 7168] -> E4M3 14.85 ->
+    // Row-wise tiles where they fit the columns exactly.  Measured on MI355X against wide tiles: bf16 [4096, 7168] -> E4M3 14.85 ->
     // 14.46 us, [32768, 4096] 59.4 -> 56.8 us, given scales 15.83 -> 15.61 us; the scale-only mode, whose only stores
     // are the scales, is better off with the staged runs of the wide tile (10.15 us against 10.85 us).
-    if (p.sf.layout == TK_SF_ROW_F32 && p.mode != TK_SF_ONLY && p.K % (RPW * kStripCols) == 0 && p.M % kWaves == 0 &&
-        tile_grid_exact(tiles_k, tiles_m))
+    if (p.sf.layout == TK_SF_ROW_F32 && p.mode != TK_SF_ONLY && p.K % (RPW * kStripCols) == 0)
         launch_per_token_tiled<InT, G, FMT, T_ROWWISE>(p, stream);
     // a caller-supplied scale tensor is only read, so either tile shape does
     else if (p.sf.layout == TK_SF_ROW_F32 && wide_tiles_pay(p.K)) launch_per_token_tiled<InT, G, FMT, T_WIDE>(p, stream);

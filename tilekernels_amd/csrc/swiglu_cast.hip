@@ -91,14 +91,18 @@ __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
 //             [32768, 2 x 2048] 60.6 -> 52.4, [16384, 2 x 4096] 69.4 -> 53.9, [8192, 2 x 6144] 48.8 -> 40.9
 //   T_STACKED (other H): 4*RPW rows x 512 columns, the 4 waves stacked; the scales are staged in LDS and stored
 //             transposed (row-major: one short run per row)
-// W = blockDim.x / 64.  FULL: the tile grid covers the matrix exactly: no bounds checks are compiled in.
+// W = blockDim.x / 64.  FULL_GRID: the tile grid covers the matrix exactly: no bounds checks are compiled in.
 // MASK: pos_to_expert is given.
 enum { T_STACKED = 0, T_ROW = 2, T_ROWC = 3 };
 
 // ONECOL: the grid is known to be a single column of tiles (else it is found out at run time)
-template <typename InT, int CLAMP, int RPW, int TILE, bool FULL, bool MASK, bool ONECOL>
+template <typename InT, int CLAMP, int RPW, int TILE, bool FULL_GRID, bool MASK, bool ONECOL>
 __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
     TK_SWIGLU_KERNEL_UNPACK;
+    // T_ROW tiles always fit the columns, and their waves share nothing: on a grid that overhangs the last row the waves
+    // beyond it leave at once and the others run without bounds checks, like on an exact grid
+    constexpr bool ROWGUARD = TILE == T_ROW && !FULL_GRID && CLAMP != 2;
+    constexpr bool FULL = FULL_GRID || ROWGUARD;
     constexpr bool ROWC = TILE == T_ROWC, ROW = TILE == T_ROW || ROWC;   // ROW: a wave's pieces lie along one row
     constexpr bool DIRECT = TILE == T_ROW;  // the wave stores its scales itself
     constexpr int GPS = kStripCols / 128;   // 4 groups per strip
@@ -127,6 +131,9 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
         const int strip = ROW ? tile_k * RPW : tile_k;
         const int col = strip * kStripCols + lane * 8;
         const int row0 = ROW ? tile_m * nwaves + wave : tile_m * ROWS + srow;
+        if constexpr (ROWGUARD) {
+            if (row0 >= p.R) return;
+        }
         const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * (2 * (int64_t)p.H) + col;
         constexpr int kRowStep = ROW ? 0 : 1, kColStep = ROW ? kStripCols : 0;
 
