@@ -707,6 +707,8 @@ def reduce_fused(x: Union[torch.Tensor, QuantTensor], topk_weights: Optional[tor
     for k in range(num_topk):
         pos = token_topk_to_pos[:, k].long()
         live = pos >= 0
+        if not bool(live.any()):
+            continue      # nothing to add (and x may have no rows at all)
         src = pos.clamp(min=0)
         s = topk_weights[:, k].clone() if topk_weights is not None else torch.ones(num_tokens, dtype=torch.float32)
         if x_sf is not None:

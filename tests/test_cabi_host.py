@@ -183,6 +183,7 @@ def test_per_channel_cast_validation(lib):
     assert check_pc(lib, K=20) == SHAPE                                 # K % 8
     assert check_pc(lib, T=128) == SHAPE                                # without a gather the input must hold M rows
     assert check_pc(lib, T=128, p2t=P) == OK
+    assert check_pc(lib, T=0, p2t=P) == SHAPE                           # a gather needs at least one input row (row 0 stands in for dropped ones)
     assert check_pc(lib, x_sf=P, K=192) == MODE                         # FP8 input comes with 1 x 128 scales
     assert check_pc(lib, x_sf=P, K=256) == OK
     assert check_pc(lib, x_sf=P, sw=1) == MODE

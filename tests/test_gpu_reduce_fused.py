@@ -63,3 +63,15 @@ def test_expand_then_reduce_is_the_weighted_identity():
     w = torch.full((T, K), 0.25, device='cuda')
     back = tk.moe.reduce_fused(tk.moe.expand_to_fused(x, t2p, p2e), w, t2p)
     assert torch.equal(back, x)          # four exact quarters of the same value
+
+
+def test_reduce_fused_without_any_live_position():
+    """Every (token, k) pair dropped: the expanded tensor has no rows; the result is zeros, as the oracle's."""
+    tk = _tk()
+    t2p = torch.full((5, 3), -1, dtype=torch.int32)
+    for dtype in (torch.bfloat16, torch.float32):
+        x = torch.empty((0, 512), dtype=dtype)
+        for fp8 in ('', 'e4m3'):
+            got = tk.moe.reduce_fused(x.cuda(), torch.rand((5, 3)).cuda(), t2p.cuda(), fp8_format=fp8)
+            want = torch_ref.reduce_fused(x, torch.rand((5, 3)), t2p, fp8_format=fp8)
+            assert_same(got, want, f'{dtype} {fp8}')

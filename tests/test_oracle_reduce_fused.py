@@ -73,3 +73,11 @@ def test_rounding_to_the_output_types():
     # the E4M3 neighbours of 1 are 1.0 and 1.125, midpoint 1.0625: 1.00195 * 1.06 = 1.06207 goes down, * 1.0625 = 1.06458 goes up
     assert torch_ref.reduce_fused(x, None, pos, 'e4m3', torch.tensor([1.06])).float()[0, 0].item() == 1.0
     assert torch_ref.reduce_fused(x, None, pos, 'e4m3', torch.tensor([1.0625])).float()[0, 0].item() == 1.125
+
+
+def test_no_live_position_at_all():
+    """Every pair dropped: the expanded tensor has no rows and the result is zeros."""
+    x = torch.empty((0, 256), dtype=torch.bfloat16)
+    t2p = torch.full((3, 2), -1, dtype=torch.int32)
+    out = torch_ref.reduce_fused(x, torch.rand((3, 2)), t2p)
+    assert out.shape == (3, 256) and out.dtype == torch.bfloat16 and torch.all(out == 0)

@@ -382,6 +382,12 @@ __global__ __launch_bounds__(kThreads) void reduce_fused_kernel(const typename R
     }
 }
 
+// reduce_fused without a single expanded row: every term is skipped, the result is zeros.  (The reduction kernel
+// cannot run then: its skipped terms read row 0, which does not exist.)
+__global__ __launch_bounds__(kThreads) void reduce_zero_kernel(uint64_t *out, int64_t words) {
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < words; i += (int64_t)gridDim.x * kThreads) out[i] = 0ull;
+}
+
 }  // namespace tk
 
 using namespace tk;
@@ -521,6 +527,13 @@ extern "C" int tk_reduce_fused(const void *x, int x_dtype, int64_t num_expanded,
                                          num_topk, out, out_dtype, sf);
     if (rc != TK_OK || num_tokens == 0) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (num_expanded == 0) {
+        const int64_t words = num_tokens * hidden * (out_dtype == TK_F32 ? 4 : (out_dtype == TK_BF16 ? 2 : 1)) / 8;   // hidden % 8 == 0
+        const int64_t blocks = (words + kThreads - 1) / kThreads;
+        hipLaunchKernelGGL(reduce_zero_kernel, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(kThreads), 0, s,
+                           static_cast<uint64_t *>(out), words);
+        return (int)hipGetLastError();
+    }
     const unsigned chunks = (unsigned)((hidden + kThreads * 8 - 1) / (kThreads * 8));
     // tokens ride on grid.y (at most 65535 per launch)
     for (int64_t t0 = 0; t0 < num_tokens; t0 += 65535) {

@@ -319,6 +319,8 @@ extern "C" int tk_check_per_channel_cast(const void *x, int x_dtype, const float
     if (num_tokens < 0 || M < 0 || K <= 0 || K % 8 != 0 || M % 16 != 0) return TK_ERR_BAD_SHAPE;
     if (x_sf && (K % 128 != 0 || swiglu)) return TK_ERR_BAD_MODE;
     if (!pos_to_token && num_tokens < M) return TK_ERR_BAD_SHAPE;
+    // gathered rows with a negative index are read from row 0 and zeroed by value, so that row must exist
+    if (pos_to_token && num_tokens == 0 && M > 0) return TK_ERR_BAD_SHAPE;
     if (swiglu && pos_to_token) return TK_ERR_BAD_MODE;
     if (use_clamp && (!swiglu || !(clamp == clamp))) return TK_ERR_BAD_VALUE;
     if (num_tokens > INT32_MAX - 256 || M > INT32_MAX - 256 || K > (INT32_MAX - 1024) / 2) return TK_ERR_TOO_LARGE;
