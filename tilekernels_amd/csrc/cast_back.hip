@@ -5,7 +5,7 @@
 // consecutive codes (8 or 4 bytes), their shared scale, and writes 16 bytes; for fp32 it takes 4 codes
 // of two pieces 256 columns apart and writes 16 bytes of each, so that every store instruction of a
 // wave covers whole cache lines.  A workgroup covers 2 rows x up to 4096 columns (row-major scales) or
-// 8 rows x 512 columns.
+// 8 rows x 512 columns; half as many rows for fp32 output.
 //
 // Reference semantics: tile_kernels/quant/cast_back_kernel.py:19-75 (kernel) and :77-143 (wrappers),
 // tile_kernels/torch/cast.py:40-59 (oracle).
@@ -16,7 +16,9 @@ namespace tk {
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kBackRowsPerWave = 2;
+// Rows per wave.  Measured on MI355X, E4M3 [8192, 4096] (us per call, 1 / 2 / 4 rows): to bf16 18.8 / 17.4 / 18.4, to fp32
+// (whose lanes already hold two pieces per row) 28.8 / 29.6 / 31.4.
+template <bool OUT_F32> constexpr int back_rows_per_wave() { return OUT_F32 ? 1 : 2; }
 
 // WIDE: the workgroup's waves stand side by side on the same RPW rows (row-major scales: one
 // workgroup then reads a row's scales once, instead of eight workgroups on eight L2s each fetching
@@ -25,7 +27,7 @@ template <typename InT, bool OUT_F32, bool WIDE, bool FULL>
 __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_back_kernel(const void *x, void *out, void *a_sf, int64_t a_sf_ld,
                                                                                          int M, int K, int geom, int bm, int bk, int a_sf_layout,
                                                                                          int nm, int nk) {
-    constexpr int RPW = kBackRowsPerWave, ROWS = WIDE ? RPW : kWaves * RPW;
+    constexpr int RPW = back_rows_per_wave<OUT_F32>(), ROWS = WIDE ? RPW : kWaves * RPW;
     const SfRef sf{a_sf, a_sf_ld, a_sf_layout, nm, nk};
     // geom: wide tiles: waves per tile, the tile index comes from the grid (x = column tile, y and z = row
     // tile); otherwise the number of column tiles of a 1-D grid
@@ -101,7 +103,8 @@ static void launch_cast_back_2(const void *x, void *out, const void *sf, int64_t
                                hipStream_t stream) {
     const int strips = (K + kStripCols - 1) / kStripCols;
     const int waves = WIDE ? wide_tile_waves(strips) : kWaves;
-    const int rows = WIDE ? kBackRowsPerWave : kWaves * kBackRowsPerWave;
+    constexpr int RPW = back_rows_per_wave<OUT_F32>();
+    const int rows = WIDE ? RPW : kWaves * RPW;
     const int cols = WIDE ? waves * kStripCols : kStripCols;
     const int tiles_m = (M + rows - 1) / rows, tiles_k = (K + cols - 1) / cols;
     const int nm = (M + bm - 1) / bm, nk = (K + bk - 1) / bk;
