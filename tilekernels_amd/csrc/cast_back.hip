@@ -98,6 +98,63 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_bac
     }
 }
 
+// Short rows: the rows laid end to end in pieces of 8 codes, lane slot L serving piece L of the sequence, so that every
+// lane has a piece whatever the row length (with 512-column strips a row of 576 columns keeps 72 of every 128 lanes
+// busy, one of 64 columns 8 of 64).  fp32 output as in the tiled kernel: a lane takes 4 codes of two pieces 32 pieces
+// apart, so that a store instruction of the wave covers consecutive bytes wherever the pieces are consecutive.
+template <typename InT, bool OUT_F32>
+__global__ __launch_bounds__(kThreads) void cast_back_flat_kernel(const void *x, void *out, void *a_sf, int64_t a_sf_ld, int M, int K, int ppr,
+                                                                  int bm, int bk, int a_sf_layout, int nm, int nk) {
+    constexpr int RPW = 2;
+    const SfRef sf{a_sf, a_sf_ld, a_sf_layout, nm, nk};
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const unsigned total = (unsigned)M * (unsigned)ppr;
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+        const unsigned slot = (unsigned)((blockIdx.x * kWaves + wave) * RPW + r);
+        if constexpr (OUT_F32) {
+            const bool hi = lane & 1;
+            Raw8<InT> raw[2];
+            int row[2], col[2];
+            bool ok[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const unsigned piece = slot * 64u + (unsigned)(h * 32 + (lane >> 1));
+                ok[h] = piece < total;
+                row[h] = (int)(piece / (unsigned)ppr);
+                col[h] = (int)(piece - (unsigned)row[h] * (unsigned)ppr) * 8;
+                raw[h].load(ok[h] ? elem_ptr<InT>(x, row[h], K, col[h]) : x);
+                raw[h].s = sf_load(sf, ok[h] ? row[h] / bm : 0, ok[h] ? col[h] / bk : 0);
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                if (!ok[h]) continue;
+                float v[4];
+                raw[h].get4(v, hi);
+                const int64_t idx = (int64_t)row[h] * K + col[h] + (hi ? 4 : 0);
+                __builtin_nontemporal_store(u32x4{f2u(v[0]), f2u(v[1]), f2u(v[2]), f2u(v[3])},
+                                            reinterpret_cast<u32x4 *>(reinterpret_cast<float *>(out) + idx));
+            }
+        } else {
+            const unsigned piece = slot * 64u + (unsigned)lane;
+            const bool ok = piece < total;
+            const int row = (int)(piece / (unsigned)ppr), col = (int)(piece - (unsigned)row * (unsigned)ppr) * 8;
+            Raw8<InT> raw;
+            raw.load(ok ? elem_ptr<InT>(x, row, K, col) : x);
+            raw.s = sf_load(sf, ok ? row / bm : 0, ok ? col / bk : 0);
+            if (!ok) continue;
+            float v[8];
+            raw.get(v);
+            u32x4 w;
+            w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[0], v[1]}), bf16x2));
+            w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[2], v[3]}), bf16x2));
+            w.z = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[4], v[5]}), bf16x2));
+            w.w = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[6], v[7]}), bf16x2));
+            __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(out) + (int64_t)row * K + col));
+        }
+    }
+}
+
 template <typename InT, bool OUT_F32, bool WIDE>
 static void launch_cast_back_2(const void *x, void *out, const void *sf, int64_t sf_ld, int M, int K, int sf_layout, int bm, int bk,
                                hipStream_t stream) {
@@ -125,6 +182,14 @@ static hipError_t launch_cast_back(const void *x, void *out, const void *sf, int
     // either way: E4M3 [8192, 4096] to bf16 17.25 -> 17.43 us, to fp32 29.63 -> 29.08 us)
     // wide tiles with column-major scales are no faster (E4M3 [8192, 4096]) and slower with 32 x 32 blocks (20.9 us
     // against 16.2 us): a 2-row tile then uses 8 bytes of each scale line it touches
+    // rows that fill less than 80 % of their 512-column strips
+    const int64_t strips = (K + kStripCols - 1) / kStripCols, pieces = (int64_t)M * (K / 8);
+    if (K * 5 < strips * kStripCols * 4 && pieces < INT32_MAX - 4 * kThreads) {   // pieces are numbered in 32 bits
+        const int64_t blocks = (pieces + 2 * kThreads - 1) / (2 * kThreads);
+        hipLaunchKernelGGL((cast_back_flat_kernel<InT, OUT_F32>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, x, out,
+                           const_cast<void *>(sf), sf_ld, M, K, K / 8, bm, bk, sf_layout, (M + bm - 1) / bm, (K + bk - 1) / bk);
+        return hipGetLastError();
+    }
     if (sf_layout == TK_SF_ROW_F32 && wide_tiles_pay(K)) launch_cast_back_2<InT, OUT_F32, true>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);
     else launch_cast_back_2<InT, OUT_F32, false>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);
     return hipGetLastError();

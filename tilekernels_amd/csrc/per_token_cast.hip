@@ -274,6 +274,81 @@ static void launch_per_token_rowgroup(PerTokenParams &p, hipStream_t stream) {
 #undef TK_ROWGROUP_LAUNCH
 }
 
+// Short rows (plain inputs): the strips of the tiled kernels are 512 columns wide, so a row of 576 columns keeps 72 of
+// every 128 lanes busy.  Here the rows are laid end to end in units of one group instead: lane slot L serves group
+// L / LPG of the sequence (row 0's groups, row 1's groups, ...), 8 elements per lane, and only the last group of a row
+// can be partly empty (576 columns in groups of 128: 72 of 80 lanes).  A wave holds RPW slots of 64 lanes; every group
+// is complete inside one slot, so the reductions and the shared scale arithmetic are those of the tiled kernel.  Each
+// scale is stored by one lane (all three layouts).
+template <typename InT, int G, int FMT, int RPW>
+__global__ __launch_bounds__(kThreads) void per_token_cast_flat_kernel(TK_PT_KERNEL_ARGS) {
+    TK_PT_KERNEL_UNPACK;
+    constexpr int LPG = G / 8;
+    using RS = RowScales<Fmt<FMT>::qmax, RPW, LPG>;
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const int gpr = p.geom;   // groups per row
+    const int64_t out_ld = FMT == TK_E4M3 ? p.K : p.K / 2;
+    const int own = lane % LPG;
+
+    int row[RPW], grp[RPW];
+    bool ok[RPW];
+    Raw8<InT> raw[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+        const unsigned slot = (unsigned)((blockIdx.x * kWaves + wave) * RPW + r);
+        const unsigned gs = (slot * 64u + (unsigned)lane) / (unsigned)LPG;
+        row[r] = (int)(gs / (unsigned)gpr);
+        grp[r] = (int)(gs - (unsigned)row[r] * (unsigned)gpr);
+        const int col = grp[r] * G + own * 8;
+        ok[r] = row[r] < p.M && col < p.K;
+        // no branch around the load: a lane beyond the matrix reads its first bytes and is cleared by value
+        raw[r].load(ok[r] ? elem_ptr<InT>(p.x, row[r], p.x_ld, col) : p.x);
+        if (!ok[r]) raw[r].zero();
+    }
+
+    float inv[RPW];
+    if (p.mode == TK_CAST_GIVEN_SF) {
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) inv[r] = 1.0f / (ok[r] ? sf_load_select(p.sf, row[r], grp[r]) : 1.0f);
+    } else {
+        float amax[RPW];
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            float v[8];
+            raw[r].get(v);
+            amax[r] = group_allmax<LPG>(absmax8(v));
+        }
+        RS rs;
+        rs.compute(amax, Fmt<FMT>::floor_, p.round_sf != 0, lane);
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) inv[r] = rs.inv[r];
+        // lane j (< A) of a group computed the scale of slot c*A + j
+        if (own < RS::A) {
+#pragma unroll
+            for (int c = 0; c < RS::NC; ++c) {
+                // the slot's row and group, chosen by value (no dynamic indexing of the arrays)
+                int m = row[c * RS::A], k = grp[c * RS::A];
+                if (RS::A >= 2 && own == 1) { m = row[c * RS::A + (RS::A >= 2 ? 1 : 0)]; k = grp[c * RS::A + (RS::A >= 2 ? 1 : 0)]; }
+                if (RS::A >= 4 && own == 2) { m = row[c * RS::A + (RS::A >= 4 ? 2 : 0)]; k = grp[c * RS::A + (RS::A >= 4 ? 2 : 0)]; }
+                if (RS::A >= 4 && own == 3) { m = row[c * RS::A + (RS::A >= 4 ? 3 : 0)]; k = grp[c * RS::A + (RS::A >= 4 ? 3 : 0)]; }
+                if (m < p.M) sf_store(p.sf, m, k, rs.own[c]);
+            }
+        }
+    }
+    if (p.mode != TK_SF_ONLY) {
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            if (!ok[r]) continue;
+            float v[8];
+            raw[r].get(v);
+            uint8_t *out_row = p.out + (int64_t)row[r] * out_ld;
+            const int col = grp[r] * G + own * 8;
+            if (p.mode == TK_CAST_GIVEN_SF) quantise_store8<FMT, true>(v, inv[r], out_row, col);
+            else quantise_store8<FMT, false>(v, inv[r], out_row, col);
+        }
+    }
+}
+
 // Rows per wave.  Measured on MI355X (us per call): bf16 [4096, 7168] -> E4M3 1x128 row-major scales
 // 18.1 / 16.3 / 17.0 for 1 / 2 / 4 rows; bf16 [16384, 7168] -> E2M1 1x32 packed scales 55.2 / 43.4 / 45.4.
 // Quantised input: a lane's 8 codes are only 8 (or 4) bytes, so a wave takes more rows to amortise
@@ -298,9 +373,27 @@ static void launch_per_token_tiled(PerTokenParams &p, hipStream_t stream) {
         hipLaunchKernelGGL((per_token_cast_kernel<InT, G, FMT, RPW, TILE, false>), grid, block, 0, stream, TK_PT_LAUNCH_ARGS(p));
 }
 
+// Whether the flattened kernel keeps more lanes busy than 512-column strips do (and the strips less than 80 %).
+inline bool short_rows_pay(int64_t K, int G) {
+    const int64_t strips = (K + kStripCols - 1) / kStripCols, groups = (K + G - 1) / G;
+    return K * 5 < strips * kStripCols * 4 && groups * G < strips * kStripCols;
+}
+
 template <typename InT, int G, int FMT>
 static void launch_per_token_group(PerTokenParams &p, hipStream_t stream) {
     constexpr int RPW = rows_per_wave<InT>();
+    if constexpr (!Elem<InT>::quantised) {
+        if (short_rows_pay(p.K, G)) {
+            const int64_t gpr = (p.K + G - 1) / G, lanes = (int64_t)p.M * gpr * (G / 8);
+            const int64_t blocks = (lanes + kThreads * RPW - 1) / (kThreads * RPW);
+            if (lanes < INT32_MAX - 2 * kThreads * RPW) {   // lane slots are numbered in 32 bits
+            p.geom = (int)gpr;
+            hipLaunchKernelGGL((per_token_cast_flat_kernel<InT, G, FMT, RPW>), dim3((unsigned)blocks), dim3(kThreads), 0, stream,
+                               TK_PT_LAUNCH_ARGS(p));
+            return;
+            }
+        }
+    }
     // Row-wise tiles where they fit the columns exactly.  Measured on MI355X against wide tiles: bf16 [4096, 7168] -> E4M3 14.85 ->
     // 14.46 us, [32768, 4096] 59.4 -> 56.8 us, given scales 15.83 -> 15.61 us; the scale-only mode, whose only stores
     // are the scales, is better off with the staged runs of the wide tile (10.15 us against 10.85 us).
