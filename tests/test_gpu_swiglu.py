@@ -49,7 +49,8 @@ def check_fused(got, want, nk, packed, what=''):
 @pytest.mark.parametrize('with_mask', [False, True])
 @pytest.mark.parametrize('H,N', [(2048, 128), (288 * 4 + 128, 128), (1024, 1024), (3584, 128), (384, 384),
                                  (512, 128), (896, 128), (5632, 128),    # one, two and eleven 512-column strips
-                                 (2560, 2560), (4224, 4224), (8192, 8192), (8320, 8320)])   # whole-row groups: 2, 3, 4 register pieces, two passes
+                                 (2560, 2560), (4224, 4224), (8192, 8192), (8320, 8320),    # whole-row groups: 2, 3, 4 register pieces, two passes
+                                 (768, 128), (256, 128)])   # short rows: laid end to end over the lanes
 def test_swiglu_forward_and_per_token_cast(H, N, with_mask, with_weights, mode, clamp):
     tk = _tk()
     col, rnd, packed = mode

@@ -239,6 +239,82 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
     counter.flush(p.clamped_count);
 }
 
+// Short rows (H fills less than 80 % of its 512-column strips: 768, 384, 256 ...): the rows laid end to end in units
+// of one 128-column group, lane slot L serving group L / 16 of the sequence, 8 outputs per lane; only the last group of
+// a row can be partly empty.  Every group is complete inside 64 lanes, so the reduction and the shared scale arithmetic
+// are those of the tiled kernel; rows differ from lane to lane, so mask and weight are read per lane, and each scale is
+// stored by one lane (all three layouts).  CLAMP: 0 none, 1 clamp (the counting variant stays with the tiled kernel).
+template <typename InT, int CLAMP, int RPW>
+__global__ __launch_bounds__(kThreads) void swiglu_cast_flat_kernel(TK_SWIGLU_KERNEL_ARGS) {
+    TK_SWIGLU_KERNEL_UNPACK;
+    constexpr int LPG = 16;
+    using RS = RowScales<448, RPW, LPG>;
+    const int lane = threadIdx.x & 63, wave = wave_id(), own = lane & 15;
+    const int gpr = p.tiles_k;   // groups per row
+    const InT *xb = reinterpret_cast<const InT *>(p.x);
+    ClampCounter<CLAMP> counter;
+
+    int row[RPW], grp[RPW];
+    bool inside[RPW], live[RPW];
+    Raw8<InT> rg[RPW], ru[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+        const unsigned slot = (unsigned)((blockIdx.x * kWaves + wave) * RPW + r);
+        const unsigned gs = (slot * 64u + (unsigned)lane) / (unsigned)LPG;
+        row[r] = (int)(gs / (unsigned)gpr);
+        grp[r] = (int)(gs - (unsigned)row[r] * (unsigned)gpr);
+        const int col = grp[r] * 128 + own * 8;
+        inside[r] = row[r] < p.R && col < p.H;
+        live[r] = row[r] < p.R && (p.pos_to_expert == nullptr || p.pos_to_expert[row[r]] >= 0);
+        // no branch around the loads: a padding row, and a lane beyond the matrix, reads its first bytes and is cleared by value
+        const bool ok = inside[r] && live[r];
+        const InT *src = ok ? xb + (int64_t)row[r] * (2 * (int64_t)p.H) + col : xb;
+        rg[r].load(src);
+        ru[r].load(ok ? src + p.H : src);
+        if (!ok) { rg[r].zero(); ru[r].zero(); }
+    }
+
+    float v[RPW][8], amax[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+        float g[8], u[8];
+        rg[r].get(g);
+        ru[r].get(u);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            counter.apply(g[i], u[i], p.clamp);
+            v[r][i] = silu_mul<InT>(g[i], u[i]);
+        }
+        if (p.pos_to_token_topk) {
+            float w = 0.0f;
+            if (live[r]) {
+                const int pos = p.pos_to_token_topk[row[r]];
+                if (pos >= 0 && pos < p.num_weights) w = p.topk_weights[pos];
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[r][i] = v[r][i] * w;
+        }
+        amax[r] = group_allmax<16>(absmax8(v[r]));
+    }
+    RS rs;
+    rs.compute(amax, p.floor_, p.round_sf != 0, lane);
+    // lane j (< A) of a group computed the scale of slot c*A + j: its row and group are chosen by value
+    if (own < RS::A) {
+#pragma unroll
+        for (int c = 0; c < RS::NC; ++c) {
+            int m = row[c * RS::A], k = grp[c * RS::A];
+            bool alive = live[c * RS::A];
+            if (RS::A >= 2 && own == 1) { m = row[c * RS::A + 1]; k = grp[c * RS::A + 1]; alive = live[c * RS::A + 1]; }
+            Scale sc = rs.own[c];
+            if (!alive) { sc.sf = 0.0f; sc.e8 = 0u; }      // padding rows carry zero scales
+            if (m < p.R) sf_store(p.sf, m, k, sc);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RPW; ++r)
+        if (inside[r]) quantise_store8<TK_E4M3, false>(v[r], live[r] ? rs.inv[r] : 0.0f, p.out + (int64_t)row[r] * p.H, grp[r] * 128 + own * 8);
+}
+
 // One scale per row (group == H): a workgroup per row.  Rows of up to ITER * 2048 outputs (ITER = 1..4) are
 // evaluated once and held in registers between the amax and the conversion; ITER == 0 takes longer rows and
 // evaluates the activation twice (amax pass, then convert pass; the second read comes from L2).  Row-major scales
@@ -386,6 +462,18 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
 template <typename InT, int CLAMP>
 static hipError_t launch_swiglu_2(SwigluParams &p, bool row_group, int max_blocks, hipStream_t stream) {
     constexpr int kPieces = swiglu_pieces<InT>();
+    if constexpr (CLAMP != 2) {
+        // rows that fill less than 80 % of their 512-column strips: [87296, 2 x 768] bf16 58.2 us tiled
+        const int64_t strips = (p.H + kStripCols - 1) / kStripCols, gpr = p.H / 128, lanes = (int64_t)p.R * gpr * 16;
+        if (!row_group && p.H * 5 < strips * kStripCols * 4 && lanes < INT32_MAX - 4 * kThreads) {
+            constexpr int RPW = 2;
+            static_assert(RowScales<448, RPW, 16>::A == 2, "the flat kernel selects between two slots");
+            p.tiles_k = (int)gpr;
+            hipLaunchKernelGGL((swiglu_cast_flat_kernel<InT, CLAMP, RPW>), dim3((unsigned)((lanes + kThreads * RPW - 1) / (kThreads * RPW))),
+                               dim3(kThreads), 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+            return hipGetLastError();
+        }
+    }
     if (row_group) {
         const int grid = max_blocks > 0 && max_blocks < p.R ? max_blocks : p.R;
         // the fewest pieces per thread (1..4) with which at most 4 waves cover a row, then the fewest waves that do
