@@ -317,6 +317,35 @@ def op_swiglu_weighted():
     return launch, algo, nbytes(x, out, sf), cpu
 
 
+def op_swiglu_dense(R, H, packed_col_major):
+    """The headline operator on dense rows of other shapes and scale layouts: packed UE8M0 column-major scales (the layout a
+    block-scaled GEMM consumes) at the headline shape, and short rows (H = 768)."""
+    def build():
+        import tilekernels_amd as tk
+        from tilekernels_amd import _ffi
+        from tilekernels_amd.quant.common import alloc_scaling_factors, get_cast_output_config, sf_leading_dim
+        lib = _ffi.load()
+        x = torch.randn((R, 2 * H), device='cuda', dtype=torch.bfloat16)
+        out = torch.empty((R, H), device='cuda', dtype=torch.float8_e4m3fn)
+        oc = get_cast_output_config('e4m3', (1, 128), packed_col_major, packed_col_major, packed_col_major)
+        sf = alloc_scaling_factors((R, H), oc, x.device)
+        stream = _ffi.current_stream(x.device)
+
+        def launch():
+            rc = lib.tk_swiglu_per_token_cast(x.data_ptr(), _ffi.TK_BF16, R, H, out.data_ptr(), sf.data_ptr(), sf_leading_dim(sf), 128,
+                                              oc.layout_code, int(packed_col_major), -1.0, 0, 0, 0, 0, 0, 0.0, 0, 0, stream)
+            assert rc == 0, rc
+        b = nbytes(x, out) + R * (H // 128) * (1 if packed_col_major else 4)
+
+        def cpu():
+            from oracle import torch_ref
+            xc = x.cpu()
+            return lambda: torch_ref.swiglu_forward_and_per_token_cast(xc, 'e4m3', 128, use_tma_aligned_col_major_sf=packed_col_major,
+                                                                       round_sf=packed_col_major, use_packed_ue8m0=packed_col_major)
+        return launch, b, b, cpu
+    return build
+
+
 def op_e5m6(direction):
     """per_token_cast(fmt='e5m6') of bf16 [8192, 4096] (one scale per row) and its dequantisation."""
     def build():
@@ -422,6 +451,10 @@ OPS = [
        op_cast_variant('block', 'given_sf')),
     Op('swiglu_forward_and_per_token_cast_weighted',
        'swiglu_forward_and_per_token_cast e4m3 1x128, MoE-expanded bf16 [R,4096] with mask and routing weights', op_swiglu_weighted),
+    Op('swiglu_forward_and_per_token_cast_packed_sf', 'swiglu_forward_and_per_token_cast e4m3 1x128, packed UE8M0 column-major scales, bf16 [8192,4096]',
+       op_swiglu_dense(8192, 2048, True)),
+    Op('swiglu_forward_and_per_token_cast_h768', 'swiglu_forward_and_per_token_cast e4m3 1x128, short rows: bf16 [32768,1536]',
+       op_swiglu_dense(32768, 768, False)),
     Op('expand_to_fused_with_sf', 'expand_to_fused_with_sf e4m3 [4096,4096] + 1x128 scales -> [R,4096], top-8 of 256 experts, pad 128',
        op_expand_to_fused_with_sf),
     Op('cast_back', 'cast_back e4m3 1x128 -> bf16, [8192,4096]', op_cast_back('bf16')),
