@@ -47,7 +47,8 @@ struct PerTokenParams {
 // Tile shapes (RPW = pieces of 8 elements per lane, i.e. of 512 columns per wave):
 //   T_WIDE    (row-major scales):      RPW rows x (W*512) columns, W = blockDim.x/64 waves side by side on the same rows;
 //             the tile's scales are RPW contiguous runs, staged in LDS and stored as whole segments
-//   T_STACKED (column-major layouts, and rows of at most 1024 columns):  4*RPW rows x 512 columns, the 4 waves stacked;
+//   T_STACKED (column-major layouts, and row lengths whose strips do not split evenly over 3..8 waves):  4*RPW rows x 512
+//             columns, the 4 waves stacked;
 //             the staged scales are stored transposed, 4*RPW rows per contiguous segment (row-major: one short run per row)
 //   T_ROWWISE (row-major scales, K a multiple of RPW*512): 4 rows x (RPW*512) columns, one row per
 //             wave; the scales a wave produces are neighbours in the scale row and it stores them itself: no LDS
