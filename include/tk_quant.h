@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define TK_QUANT_VERSION 109 /* major*10000 + minor*100 + patch */
+#define TK_QUANT_VERSION 110 /* major*10000 + minor*100 + patch */
 
 enum tk_dtype { TK_BF16 = 0, TK_F32 = 1, TK_OUT_E4M3 = 2 /* output of tk_reduce_fused only */ };
 enum tk_fmt { TK_E4M3 = 0, TK_E2M1 = 1, TK_E5M6 = 2 };
@@ -192,7 +192,8 @@ int tk_check_swiglu_backward_per_token_cast(const void *x, const float *x_sf, in
  *   swiglu != 0               : bf16 x[num_tokens, 2K]; the value cast is bf16(g / (1 + exp(-g)) * u) with
  *                               g = x[:, :K], u = x[:, K:], clamped as in tk_swiglu_per_token_cast with use_clamp
  * pos_to_token (NULL, or int32[M]) gathers rows: output row r comes from input row pos_to_token[r], a
- * negative index gives a row of zeros; without it M rows are taken in order (num_tokens >= M).
+ * negative index gives a row of zeros; without it M rows are taken in order (num_tokens >= M).  A gather needs
+ * num_tokens >= 1 (TK_ERR_BAD_SHAPE otherwise).
  * transpose == 0: out[M, K];  transpose != 0: out[K, M].
  * Stands behind tile_kernels.quant.per_channel_cast, per_channel_cast_fused
  * (tile_kernels/quant/per_channel_cast_fused_kernel.py:130-203), per_channel_cast_and_transpose
@@ -213,7 +214,8 @@ int tk_check_per_channel_cast(const void *x, int x_dtype, const float *x_sf, int
  *   out[t, :] = round( sf * sum_k  x[pos, :] * (topk_weights[t, k] * x_sf[pos]) ),   pos = token_topk_to_pos[t, k] >= 0
  * accumulated in fp32 with one fused multiply-add per term, k ascending; topk_weights, x_sf ([num_expanded]
  * fp32) and sf (one fp32 on the device) may each be NULL (factor 1).  x: bf16 or fp32 [num_expanded, hidden],
- * contiguous; out: the type of x, or E4M3 bytes with out_dtype = TK_OUT_E4M3.
+ * contiguous; out: the type of x, or E4M3 bytes with out_dtype = TK_OUT_E4M3.  Positions outside [0, num_expanded) are
+ * skipped; with num_expanded == 0 (x may then be NULL) the result is zeros.
  * Stands behind tile_kernels.moe.reduce_fused (tile_kernels/moe/reduce_fused_kernel.py:70-135; oracle
  * tile_kernels/torch/reduce_fused.py:14-72).
  *   requirements hidden % 8 == 0; x and out 16-byte (E4M3 out: 8-byte) aligned
