@@ -104,7 +104,7 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_bac
 // apart, so that a store instruction of the wave covers consecutive bytes wherever the pieces are consecutive.
 template <typename InT, bool OUT_F32>
 __global__ __launch_bounds__(kThreads) void cast_back_flat_kernel(const void *x, void *out, void *a_sf, int64_t a_sf_ld, int M, int K, int ppr,
-                                                                  int bm, int bk, int a_sf_layout, int nm, int nk) {
+                                                                  unsigned ppr_recip, int bm, int bk, int a_sf_layout, int nm, int nk) {
     constexpr int RPW = 2;
     const SfRef sf{a_sf, a_sf_ld, a_sf_layout, nm, nk};
     const int lane = threadIdx.x & 63, wave = wave_id();
@@ -121,8 +121,11 @@ __global__ __launch_bounds__(kThreads) void cast_back_flat_kernel(const void *x,
             for (int h = 0; h < 2; ++h) {
                 const unsigned piece = slot * 64u + (unsigned)(h * 32 + (lane >> 1));
                 ok[h] = piece < total;
-                row[h] = (int)(piece / (unsigned)ppr);
-                col[h] = (int)(piece - (unsigned)row[h] * (unsigned)ppr) * 8;
+                // piece / ppr by multiplication: with floor(2^32 / ppr) the quotient comes out exact or one too small
+                unsigned q = __umulhi(piece, ppr_recip), rem = piece - q * (unsigned)ppr;
+                if (rem >= (unsigned)ppr) { ++q; rem -= (unsigned)ppr; }
+                row[h] = (int)q;
+                col[h] = (int)rem * 8;
                 raw[h].load(ok[h] ? elem_ptr<InT>(x, row[h], K, col[h]) : x);
                 raw[h].s = sf_load(sf, ok[h] ? row[h] / bm : 0, ok[h] ? col[h] / bk : 0);
             }
@@ -138,7 +141,9 @@ __global__ __launch_bounds__(kThreads) void cast_back_flat_kernel(const void *x,
         } else {
             const unsigned piece = slot * 64u + (unsigned)lane;
             const bool ok = piece < total;
-            const int row = (int)(piece / (unsigned)ppr), col = (int)(piece - (unsigned)row * (unsigned)ppr) * 8;
+            unsigned q = __umulhi(piece, ppr_recip), rem = piece - q * (unsigned)ppr;
+            if (rem >= (unsigned)ppr) { ++q; rem -= (unsigned)ppr; }
+            const int row = (int)q, col = (int)rem * 8;
             Raw8<InT> raw;
             raw.load(ok ? elem_ptr<InT>(x, row, K, col) : x);
             raw.s = sf_load(sf, ok ? row / bm : 0, ok ? col / bk : 0);
@@ -187,7 +192,8 @@ static hipError_t launch_cast_back(const void *x, void *out, const void *sf, int
     if (K * 5 < strips * kStripCols * 4 && pieces < INT32_MAX - 4 * kThreads) {   // pieces are numbered in 32 bits
         const int64_t blocks = (pieces + 2 * kThreads - 1) / (2 * kThreads);
         hipLaunchKernelGGL((cast_back_flat_kernel<InT, OUT_F32>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, x, out,
-                           const_cast<void *>(sf), sf_ld, M, K, K / 8, bm, bk, sf_layout, (M + bm - 1) / bm, (K + bk - 1) / bk);
+                           const_cast<void *>(sf), sf_ld, M, K, K / 8,
+                           (unsigned)(K == 8 ? 0xFFFFFFFFull : (1ull << 32) / (uint64_t)(K / 8)), bm, bk, sf_layout, (M + bm - 1) / bm, (K + bk - 1) / bk);
         return hipGetLastError();
     }
     if (sf_layout == TK_SF_ROW_F32 && wide_tiles_pay(K)) launch_cast_back_2<InT, OUT_F32, true>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);

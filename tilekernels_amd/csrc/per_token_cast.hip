@@ -298,8 +298,11 @@ __global__ __launch_bounds__(kThreads) void per_token_cast_flat_kernel(TK_PT_KER
     for (int r = 0; r < RPW; ++r) {
         const unsigned slot = (unsigned)((blockIdx.x * kWaves + wave) * RPW + r);
         const unsigned gs = (slot * 64u + (unsigned)lane) / (unsigned)LPG;
-        row[r] = (int)(gs / (unsigned)gpr);
-        grp[r] = (int)(gs - (unsigned)row[r] * (unsigned)gpr);
+        // gs / gpr by multiplication: with floor(2^32 / gpr) the quotient comes out exact or one too small
+        unsigned q = __umulhi(gs, (unsigned)p.in_bm), rem = gs - q * (unsigned)gpr;
+        if (rem >= (unsigned)gpr) { ++q; rem -= (unsigned)gpr; }
+        row[r] = (int)q;
+        grp[r] = (int)rem;
         const int col = grp[r] * G + own * 8;
         ok[r] = row[r] < p.M && col < p.K;
         // no branch around the load: a lane beyond the matrix reads its first bytes and is cleared by value
@@ -389,6 +392,7 @@ static void launch_per_token_group(PerTokenParams &p, hipStream_t stream) {
             const int64_t blocks = (lanes + kThreads * RPW - 1) / (kThreads * RPW);
             if (lanes < INT32_MAX - 2 * kThreads * RPW) {   // lane slots are numbered in 32 bits
             p.geom = (int)gpr;
+            p.in_bm = (int)(uint32_t)(gpr == 1 ? 0xFFFFFFFFull : (1ull << 32) / (uint64_t)gpr);   // plain input: the field carries the reciprocal of gpr
             hipLaunchKernelGGL((per_token_cast_flat_kernel<InT, G, FMT, RPW>), dim3((unsigned)blocks), dim3(kThreads), 0, stream,
                                TK_PT_LAUNCH_ARGS(p));
             return;

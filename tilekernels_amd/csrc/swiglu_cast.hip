@@ -261,8 +261,11 @@ __global__ __launch_bounds__(kThreads) void swiglu_cast_flat_kernel(TK_SWIGLU_KE
     for (int r = 0; r < RPW; ++r) {
         const unsigned slot = (unsigned)((blockIdx.x * kWaves + wave) * RPW + r);
         const unsigned gs = (slot * 64u + (unsigned)lane) / (unsigned)LPG;
-        row[r] = (int)(gs / (unsigned)gpr);
-        grp[r] = (int)(gs - (unsigned)row[r] * (unsigned)gpr);
+        // gs / gpr by multiplication: with floor(2^32 / gpr) the quotient comes out exact or one too small
+        unsigned q = __umulhi(gs, (unsigned)p.nwaves), rem = gs - q * (unsigned)gpr;
+        if (rem >= (unsigned)gpr) { ++q; rem -= (unsigned)gpr; }
+        row[r] = (int)q;
+        grp[r] = (int)rem;
         const int col = grp[r] * 128 + own * 8;
         inside[r] = row[r] < p.R && col < p.H;
         live[r] = row[r] < p.R && (p.pos_to_expert == nullptr || p.pos_to_expert[row[r]] >= 0);
@@ -469,6 +472,7 @@ static hipError_t launch_swiglu_2(SwigluParams &p, bool row_group, int max_block
             constexpr int RPW = 2;   // slots per wave; [32768, 2 x 768] bf16: 24.1 / 23.7 / 30.6 us with 1 / 2 / 4
             static_assert(RowScales<448, RPW, 16>::A == 2, "the flat kernel selects between two slots");
             p.tiles_k = (int)gpr;
+            p.nwaves = (int)(uint32_t)(gpr == 1 ? 0xFFFFFFFFull : (1ull << 32) / (uint64_t)gpr);   // reciprocal of gpr for the kernel's divisions
             hipLaunchKernelGGL((swiglu_cast_flat_kernel<InT, CLAMP, RPW>), dim3((unsigned)((lanes + kThreads * RPW - 1) / (kThreads * RPW))),
                                dim3(kThreads), 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
             return hipGetLastError();
