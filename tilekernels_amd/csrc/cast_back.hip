@@ -104,8 +104,11 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_bac
 // apart, so that a store instruction of the wave covers consecutive bytes wherever the pieces are consecutive.
 template <typename InT, bool OUT_F32>
 __global__ __launch_bounds__(kThreads) void cast_back_flat_kernel(const void *x, void *out, void *a_sf, int64_t a_sf_ld, int M, int K, int ppr,
-                                                                  unsigned ppr_recip, int bm, int bk, int a_sf_layout, int nm, int nk) {
+                                                                  unsigned ppr_recip, int bm, int bk, int a_sf_layout, int nm, int nk, int bm_sh, int bk_sh) {
     constexpr int RPW = 2;
+    // block indices by shifts where the block extents are powers of two (bm_sh, bk_sh >= 0), which they nearly always are
+    auto blk_m = [&](int row) { return bm_sh >= 0 ? row >> bm_sh : row / bm; };
+    auto blk_k = [&](int col) { return bk_sh >= 0 ? col >> bk_sh : col / bk; };
     const SfRef sf{a_sf, a_sf_ld, a_sf_layout, nm, nk};
     const int lane = threadIdx.x & 63, wave = wave_id();
     const unsigned total = (unsigned)M * (unsigned)ppr;
@@ -127,7 +130,7 @@ __global__ __launch_bounds__(kThreads) void cast_back_flat_kernel(const void *x,
                 row[h] = (int)q;
                 col[h] = (int)rem * 8;
                 raw[h].load(ok[h] ? elem_ptr<InT>(x, row[h], K, col[h]) : x);
-                raw[h].s = sf_load(sf, ok[h] ? row[h] / bm : 0, ok[h] ? col[h] / bk : 0);
+                raw[h].s = sf_load(sf, ok[h] ? blk_m(row[h]) : 0, ok[h] ? blk_k(col[h]) : 0);
             }
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
@@ -146,7 +149,7 @@ __global__ __launch_bounds__(kThreads) void cast_back_flat_kernel(const void *x,
             const int row = (int)q, col = (int)rem * 8;
             Raw8<InT> raw;
             raw.load(ok ? elem_ptr<InT>(x, row, K, col) : x);
-            raw.s = sf_load(sf, ok ? row / bm : 0, ok ? col / bk : 0);
+            raw.s = sf_load(sf, ok ? blk_m(row) : 0, ok ? blk_k(col) : 0);
             if (!ok) continue;
             float v[8];
             raw.get(v);
@@ -180,6 +183,13 @@ static void launch_cast_back_2(const void *x, void *out, const void *sf, int64_t
         hipLaunchKernelGGL((cast_back_kernel<InT, OUT_F32, WIDE, false>), grid, block, 0, stream, x, out, sfp, sf_ld, M, K, geom, bm, bk, sf_layout, nm, nk);
 }
 
+// log2 of a power of two, -1 for any other value
+inline int log2_or_minus1(int v) {
+    for (int s = 0; s < 31; ++s)
+        if ((1 << s) == v) return s;
+    return -1;
+}
+
 template <typename InT, bool OUT_F32>
 static hipError_t launch_cast_back(const void *x, void *out, const void *sf, int64_t sf_ld, int M, int K, int sf_layout,
                                    int bm, int bk, hipStream_t stream) {
@@ -193,7 +203,8 @@ static hipError_t launch_cast_back(const void *x, void *out, const void *sf, int
         const int64_t blocks = (pieces + 2 * kThreads - 1) / (2 * kThreads);
         hipLaunchKernelGGL((cast_back_flat_kernel<InT, OUT_F32>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, x, out,
                            const_cast<void *>(sf), sf_ld, M, K, K / 8,
-                           (unsigned)(K == 8 ? 0xFFFFFFFFull : (1ull << 32) / (uint64_t)(K / 8)), bm, bk, sf_layout, (M + bm - 1) / bm, (K + bk - 1) / bk);
+                           (unsigned)(K == 8 ? 0xFFFFFFFFull : (1ull << 32) / (uint64_t)(K / 8)), bm, bk, sf_layout, (M + bm - 1) / bm, (K + bk - 1) / bk,
+                           log2_or_minus1(bm), log2_or_minus1(bk));
         return hipGetLastError();
     }
     if (sf_layout == TK_SF_ROW_F32 && wide_tiles_pay(K)) launch_cast_back_2<InT, OUT_F32, true>(x, out, sf, sf_ld, M, K, sf_layout, bm, bk, stream);
