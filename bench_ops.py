@@ -221,6 +221,42 @@ def op_per_channel(mode, transpose, num_per_tokens=128, rows=8192, hidden=4096):
     return build
 
 
+def op_short_rows(direction):
+    """Rows of 576 columns (the shortest row length of the reference's test list): per_token_cast 1x64 and its dequantisation."""
+    def build():
+        import tilekernels_amd as tk
+        from tilekernels_amd import _ffi
+        lib = _ffi.load()
+        M, K, N = 65536, 576, 64
+        x = torch.randn((M, K), device='cuda', dtype=torch.bfloat16)
+        codes = torch.empty((M, K), device='cuda', dtype=torch.float8_e4m3fn)
+        sf = torch.empty((M, K // N), device='cuda', dtype=torch.float32)
+        back = torch.empty((M, K), device='cuda', dtype=torch.bfloat16)
+        stream = _ffi.current_stream(x.device)
+
+        def cast():
+            rc = lib.tk_per_token_cast(x.data_ptr(), _ffi.TK_BF16, M, K, K, codes.data_ptr(), sf.data_ptr(), K // N, _ffi.TK_E4M3, N,
+                                       _ffi.TK_SF_ROW_F32, 0, _ffi.TK_CAST_AND_SF, stream)
+            assert rc == 0, rc
+        cast()
+
+        def dequant():
+            rc = lib.tk_cast_back(codes.data_ptr(), _ffi.TK_E4M3, M, K, sf.data_ptr(), K // N, _ffi.TK_SF_ROW_F32, 1, N, back.data_ptr(),
+                                  _ffi.TK_BF16, stream)
+            assert rc == 0, rc
+        b = nbytes(x, codes, sf)
+
+        def cpu():
+            from oracle import torch_ref
+            xc = x.cpu()
+            if direction == 'cast':
+                return lambda: torch_ref.cast(xc, 'e4m3', (1, N))
+            q = (codes.cpu(), sf.cpu())
+            return lambda: torch_ref.cast_back(q, 'bf16', (1, N))
+        return (cast if direction == 'cast' else dequant), b, b, cpu
+    return build
+
+
 def op_cast_variant(kind, mode):
     """The scale-only and given-scale variants of the two casts at their benchmark shapes.
     kind: 'token' (bf16 [4096,7168], 1x128) or 'block' (bf16 [7168,2048], 128x128); mode: 'sf_only' or 'given_sf'."""
@@ -443,6 +479,8 @@ OPS = [
     Op('per_block_cast_lossless', 'per_block_cast_lossless e2m1 1x32 (packed scales) -> e4m3 128x128, [7168,2048]', op_lossless),
     Op('per_token_cast_e5m6', "per_token_cast fmt='e5m6' (12-bit, one scale per row) round_sf, bf16 [8192,4096]", op_e5m6('cast')),
     Op('cast_back_e5m6', 'cast_back of e5m6 -> bf16, [8192,4096]', op_e5m6('back')),
+    Op('per_token_cast_k576', 'per_token_cast e4m3 1x64, short rows: bf16 [65536,576]', op_short_rows('cast')),
+    Op('cast_back_k576', 'cast_back e4m3 1x64 -> bf16, short rows: [65536,576]', op_short_rows('back')),
     Op('per_token_cast_with_sf_only', 'per_token_cast_with_sf_only e4m3 1x128, bf16 [4096,7168]', op_cast_variant('token', 'sf_only')),
     Op('per_token_cast_with_precomputed_sf', 'per_token_cast_with_precomputed_sf e4m3 1x128, bf16 [4096,7168]',
        op_cast_variant('token', 'given_sf')),
