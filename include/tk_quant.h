@@ -286,6 +286,23 @@ int tk_check_get_fused_mapping(const int64_t *topk_idx, int64_t num_tokens, int 
                                const int32_t *num_tokens_per_expert, const void *workspace, int64_t workspace_bytes);
 
 /*
+ * tk_get_fused_mapping_static: tk_get_fused_mapping without the workspace argument, for callers that cannot
+ * allocate device memory or carry a workspace around (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid allocation).  It has no counterpart in the reference.  The slice x expert table lives
+ * in a device array of TK_FUSED_MAPPING_STATIC_BYTES bytes that the library holds on every GPU it runs on until
+ * the process ends; the call allocates and frees nothing.  Inputs whose table would not fit
+ * (tk_fused_mapping_workspace_bytes() > TK_FUSED_MAPPING_STATIC_BYTES, i.e. more than 1 Mi (token, k) pairs at
+ * 256 experts) are rejected with TK_ERR_TOO_LARGE.  Same outputs, bit for bit, as tk_get_fused_mapping.
+ * All calls on one GPU share that GPU's table: calls that overlap there (two streams, two threads) race.
+ * The first call on a device looks up the array's address and should happen outside graph capture.
+ */
+#define TK_FUSED_MAPPING_STATIC_BYTES (4 << 20)
+int tk_get_fused_mapping_static(const int64_t *topk_idx, int64_t num_tokens, int num_topk, int num_experts, int alignment,
+                                int64_t num_expanded, int32_t *pos_to_expert, int32_t *pos_to_token,
+                                int32_t *pos_to_token_topk, int32_t *token_topk_to_pos, int32_t *expert_start,
+                                int32_t *expert_end, int32_t *num_tokens_per_expert, void *stream);
+
+/*
  * tk_expand_to_fused: row t of x (row_bytes bytes, any element type) is copied to every position
  * token_topk_to_pos[t * num_topk + k] >= 0; rows with pos_to_expert < 0 are zero-filled.  With
  * x_sf != NULL the token's `sf_cols` 4-byte scale words (contiguous rows) are expanded the same way

@@ -269,6 +269,9 @@ def test_launching_entry_points_reject_before_touching_the_device(lib):
     assert lib.tk_per_block_cast(P, 0, 64, 512, P, P, 4, 0, 64, 64, 0, 0, 0, None) == GROUP
     assert lib.tk_swiglu_per_token_cast(P, 0, 64, 2000, P, P, 16, 128, 0, 0, -1.0, None, None, 0, None, 0, 0.0, None, 0, None) == SHAPE
     assert lib.tk_per_token_cast(None, 0, 0, 1024, 1024, None, None, 8, 0, 128, 0, 0, 0, None) == OK     # M == 0
+    # the entry point with library-owned scratch refuses what its table cannot hold before any device call
+    assert lib.tk_fused_mapping_workspace_bytes(262145, 4, 1024) > (4 << 20)
+    assert lib.tk_get_fused_mapping_static(P, 262145, 4, 1024, 16, 1 << 20, P, P, P, P, P, P, P, None) == LARGE
 
 
 def test_host_side_geometry_matches_the_oracle_layouts():

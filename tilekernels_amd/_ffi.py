@@ -39,6 +39,7 @@ SIGNATURES = {
     'tk_check_reduce_fused': (_i32, [_vp, _i32, _i64, _i64, _vp, _vp, _vp, _i64, _i32, _vp, _i32, _vp]),
     'tk_fused_mapping_workspace_bytes': (_i64, [_i64, _i32, _i32]),
     'tk_get_fused_mapping': (_i32, [_vp, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    'tk_get_fused_mapping_static': (_i32, [_vp, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     'tk_check_get_fused_mapping': (_i32, [_vp, _i64, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64]),
     'tk_expand_to_fused': (_i32, [_vp, _i64, _i64, _vp, _i32, _vp, _i64, _vp, _vp, _i32, _vp, _i64, _i32, _vp]),
     'tk_check_expand_to_fused': (_i32, [_vp, _i64, _i64, _vp, _i32, _vp, _i64, _vp, _vp, _i32, _vp, _i64, _i32]),

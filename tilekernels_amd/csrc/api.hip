@@ -13,7 +13,7 @@ extern "C" const char *tk_strerror(int status) {
         case TK_ERR_BAD_MODE: return "mode not usable with these options";
         case TK_ERR_BAD_STRIDE: return "row stride or scale-factor leading dimension too small";
         case TK_ERR_MISALIGNED: return "pointer or stride not aligned for vector access";
-        case TK_ERR_TOO_LARGE: return "problem too large for 32-bit tile indexing";
+        case TK_ERR_TOO_LARGE: return "problem too large for 32-bit tile indexing or for the library's static scratch";
         case TK_ERR_BAD_VALUE: return "clamp or floor value not usable";
         default: return status > 0 ? "hip error" : "unknown status";
     }

@@ -5,6 +5,8 @@
 // Reference semantics: tile_kernels/moe/get_fused_mapping_kernel.py:24-250,
 // tile_kernels/moe/expand_to_fused_kernel.py:16-200, tile_kernels/torch/expand_to_fused.py,
 // tile_kernels/moe/reduce_fused_kernel.py:12-135, tile_kernels/torch/reduce_fused.py.
+#include <atomic>
+
 #include "tk_device.hpp"
 #include "tk_host.hpp"
 
@@ -417,20 +419,14 @@ extern "C" int tk_check_get_fused_mapping(const int64_t *topk_idx, int64_t num_t
     return TK_OK;
 }
 
-extern "C" int tk_get_fused_mapping(const int64_t *topk_idx, int64_t num_tokens, int num_topk, int num_experts, int alignment,
-                                    int64_t num_expanded, int32_t *pos_to_expert, int32_t *pos_to_token,
-                                    int32_t *pos_to_token_topk, int32_t *token_topk_to_pos, int32_t *expert_start,
-                                    int32_t *expert_end, int32_t *num_tokens_per_expert, void *workspace,
-                                    int64_t workspace_bytes, void *stream) {
-    const int rc = tk_check_get_fused_mapping(topk_idx, num_tokens, num_topk, num_experts, alignment, num_expanded, pos_to_expert,
-                                              pos_to_token, pos_to_token_topk, token_topk_to_pos, expert_start, expert_end,
-                                              num_tokens_per_expert, workspace, workspace_bytes);
-    if (rc != TK_OK) return rc;
-    hipStream_t s = static_cast<hipStream_t>(stream);
+// the three launches; `ws` holds at least tk_fused_mapping_workspace_bytes() bytes
+static int launch_fused_mapping(const int64_t *topk_idx, int64_t num_tokens, int num_topk, int num_experts, int alignment,
+                                int64_t num_expanded, int32_t *pos_to_expert, int32_t *pos_to_token, int32_t *pos_to_token_topk,
+                                int32_t *token_topk_to_pos, int32_t *expert_start, int32_t *expert_end,
+                                int32_t *num_tokens_per_expert, int32_t *ws, hipStream_t s) {
     const int numel = (int)(num_tokens * num_topk);
     const int slices = (numel + kSliceElems - 1) / kSliceElems;
     const int blocks = (slices + kWaves - 1) / kWaves;
-    int32_t *ws = static_cast<int32_t *>(workspace);
     const size_t lds = (size_t)kWaves * num_experts * sizeof(int32_t);
     int bits = 0;
     while ((1 << bits) < num_experts) ++bits;
@@ -447,6 +443,69 @@ extern "C" int tk_get_fused_mapping(const int64_t *topk_idx, int64_t num_tokens,
                            bits, ws, expert_start, pos_to_expert, pos_to_token, pos_to_token_topk, token_topk_to_pos,
                            (int)num_expanded);
     return (int)hipGetLastError();
+}
+
+extern "C" int tk_get_fused_mapping(const int64_t *topk_idx, int64_t num_tokens, int num_topk, int num_experts, int alignment,
+                                    int64_t num_expanded, int32_t *pos_to_expert, int32_t *pos_to_token,
+                                    int32_t *pos_to_token_topk, int32_t *token_topk_to_pos, int32_t *expert_start,
+                                    int32_t *expert_end, int32_t *num_tokens_per_expert, void *workspace,
+                                    int64_t workspace_bytes, void *stream) {
+    const int rc = tk_check_get_fused_mapping(topk_idx, num_tokens, num_topk, num_experts, alignment, num_expanded, pos_to_expert,
+                                              pos_to_token, pos_to_token_topk, token_topk_to_pos, expert_start, expert_end,
+                                              num_tokens_per_expert, workspace, workspace_bytes);
+    if (rc != TK_OK) return rc;
+    return launch_fused_mapping(topk_idx, num_tokens, num_topk, num_experts, alignment, num_expanded, pos_to_expert, pos_to_token,
+                                pos_to_token_topk, token_topk_to_pos, expert_start, expert_end, num_tokens_per_expert,
+                                static_cast<int32_t *>(workspace), static_cast<hipStream_t>(stream));
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same mapping for callers that cannot allocate or pass a workspace: the slice x expert table lives in a
+// device array owned by the library.  Every GPU holds its own copy of the array at its own address, which is
+// looked up once per device (the array's name is only a host-side handle, never a device address) and passed
+// to the kernels like the caller's workspace above.  The count launch writes every table entry the later
+// launches read, so nothing has to be cleared between calls; calls that overlap on one GPU would share the
+// table and race.
+static __device__ __align__(256) unsigned char scratch[TK_FUSED_MAPPING_STATIC_BYTES];
+
+// device address of `scratch` on the current device
+static int static_scratch_address(void **out) {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<void *> known[kMaxDevices];
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return TK_ERR_TOO_LARGE;
+    void *ptr = known[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!ptr) return TK_ERR_NULL_POINTER;
+        known[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return TK_OK;
+}
+
+extern "C" int tk_get_fused_mapping_static(const int64_t *topk_idx, int64_t num_tokens, int num_topk, int num_experts,
+                                           int alignment, int64_t num_expanded, int32_t *pos_to_expert, int32_t *pos_to_token,
+                                           int32_t *pos_to_token_topk, int32_t *token_topk_to_pos, int32_t *expert_start,
+                                           int32_t *expert_end, int32_t *num_tokens_per_expert, void *stream) {
+    // sizes first, so that an oversized request is reported as such whatever else is wrong with it
+    if (num_tokens >= 0 && num_topk > 0 && num_experts > 0 && num_experts <= kMaxExperts &&
+        num_tokens * num_topk <= INT32_MAX - 1024 &&
+        tk_fused_mapping_workspace_bytes(num_tokens, num_topk, num_experts) > (int64_t)TK_FUSED_MAPPING_STATIC_BYTES)
+        return TK_ERR_TOO_LARGE;
+    void *ws = nullptr;
+    int rc = static_scratch_address(&ws);
+    if (rc != TK_OK) return rc;
+    rc = tk_check_get_fused_mapping(topk_idx, num_tokens, num_topk, num_experts, alignment, num_expanded, pos_to_expert,
+                                    pos_to_token, pos_to_token_topk, token_topk_to_pos, expert_start, expert_end,
+                                    num_tokens_per_expert, ws, (int64_t)TK_FUSED_MAPPING_STATIC_BYTES);
+    if (rc != TK_OK) return rc;
+    return launch_fused_mapping(topk_idx, num_tokens, num_topk, num_experts, alignment, num_expanded, pos_to_expert, pos_to_token,
+                                pos_to_token_topk, token_topk_to_pos, expert_start, expert_end, num_tokens_per_expert,
+                                static_cast<int32_t *>(ws), static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tk_check_expand_to_fused(const void *x, int64_t num_tokens, int64_t row_bytes, const int32_t *token_topk_to_pos,
