@@ -13,7 +13,15 @@ One JSON line goes to stdout.  `value` is algorithmic bytes (input read + codes 
 written) per wall-clock second over the timed region; `roofline.achieved` is the same byte count
 over the kernel's mean duration taken with HIP events on the launch stream.  `cpu_baseline` times
 the CPU oracle (test infrastructure, a restatement of the reference's torch implementation) on the
-host cores for the same workload and doubles as the in-run parity check.
+host cores for the same workload and doubles as the in-run parity check.  `configs` holds the same
+figures, in short, for the other four benchmark configurations, and `same_traffic_reference` the time
+of a stock PyTorch elementwise kernel that moves the same bytes (no arithmetic to speak of) on the same
+buffers, next to the time per launch of this entry point on a four-row input (what a launch costs on
+this stack whatever its size).
+
+Before the `--warmup` launches the GPU is kept busy with the same launches for `--preheat-ms`
+milliseconds (untimed): its clocks need about 15 ms of load to settle, and a handful of 15 us
+launches does not provide that.
 """
 import argparse
 import json
@@ -45,6 +53,24 @@ WORKLOADS = {
 }
 
 
+def algorithmic_bytes(cfg: int, data: dict) -> int:
+    """Bytes the operator of configuration `cfg` has to move for the input `data` (make_baseline_input): the input
+    read once, codes and scales written once.  Configuration 4 reads only the rows that are not padding, plus the
+    4-byte mask entry of every row, and writes zero codes and scales for the padding rows."""
+    x = data['x']
+    M = x.shape[0]
+    if cfg in (1, 5):
+        K = x.shape[1]
+        group, code_bytes, sf_bytes = (128, M * K, 4) if cfg == 1 else (32, M * K // 2, 1)
+        return x.numel() * 2 + code_bytes + M * (K // group) * sf_bytes
+    if cfg == 2:
+        K = x.shape[1]
+        return x.numel() * 2 + M * K + (M // 128) * (K // 128) * 4
+    H = x.shape[1] // 2
+    live = M if cfg == 3 else int((data['pos_to_expert'] >= 0).sum())
+    return live * 4 * H + (0 if cfg == 3 else 4 * M) + M * H + M * (H // 128) * 4
+
+
 class Workload:
     """Device buffers and the C-ABI launch closure of one benchmark configuration."""
 
@@ -66,19 +92,15 @@ class Workload:
             kw = {} if cfg == 1 else dict(use_tma_aligned_col_major_sf=True, round_sf=True, use_packed_ue8m0=True)
             oc = get_cast_output_config(fmt, (1, group), **kw)
             out_shape = (M, K if cfg == 1 else K // 2)
-            self.bytes = x.numel() * 2 + out_shape[0] * out_shape[1] + M * (K // group) * (4 if cfg == 1 else 1)
         elif cfg == 2:
             K = x.shape[1]
             oc = get_cast_output_config('e4m3', (128, 128))
             out_shape = (M, K)
-            self.bytes = x.numel() * 2 + M * K + (M // 128) * (K // 128) * 4
         else:
             H = x.shape[1] // 2
             oc = get_cast_output_config('e4m3', (1, 128))
             out_shape = (M, H)
-            live = M if cfg == 3 else int((data['pos_to_expert'] >= 0).sum())
-            # padding rows are not read; their zero codes and scales are written
-            self.bytes = live * 4 * H + (0 if cfg == 3 else 4 * M) + M * H + M * (H // 128) * 4
+        self.bytes = algorithmic_bytes(cfg, data)
         self.oc = oc
         set_bytes = x.numel() * 2 + out_shape[0] * out_shape[1]
         self.nsets = max(nsets_min, -(-int(1.6 * LLC_BYTES) // set_bytes))
@@ -113,6 +135,14 @@ class Workload:
         if rc != 0:
             raise RuntimeError(f'launch failed with status {rc}')
 
+    def small_launch(self, stream: int) -> None:
+        """The same entry point on the first four rows (128 for the per-block cast) of buffer set 0."""
+        fn, args = self.calls[0]
+        rows = 128 if self.cfg == 2 else 4
+        rc = fn(*(args[:2] + (rows,) + args[3:-1] + (stream,)))      # the row count is the third argument, the stream the last
+        if rc != 0:
+            raise RuntimeError(f'launch failed with status {rc}')
+
     def result(self, i: int = 0):
         """(codes, scales) of buffer set i as the public API would return them."""
         from tilekernels_amd.quant.common import cast_epilogue
@@ -121,7 +151,25 @@ class Workload:
         return self.out[i], cast_epilogue(self.sf[i], x.shape[0], hidden, self.oc)
 
 
-def time_gpu(w: Workload, steps: int, warmup: int):
+def preheat(w: 'Workload', ms: float) -> float:
+    """Untimed launches for at least `ms` milliseconds of GPU time; returns the milliseconds spent."""
+    if ms <= 0:
+        return 0.0
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    per_batch = max(16, int(2000.0 / (w.bytes / 6e6)))     # about 2 ms of launches per batch at 6 TB/s
+    spent, i = 0.0, 0
+    e0.record()
+    while spent < ms:
+        for _ in range(per_batch):
+            w.launch(i)
+            i += 1
+        e1.record()
+        e1.synchronize()
+        spent = e0.elapsed_time(e1)
+    return spent
+
+
+def time_gpu(w: 'Workload', steps: int, warmup: int):
     """Returns (wall seconds for `steps` launches, HIP-event microseconds per launch over the same
     timed region, list of single-launch durations from per-launch event pairs)."""
     for i in range(warmup):
@@ -133,8 +181,10 @@ def time_gpu(w: Workload, steps: int, warmup: int):
     for i in range(steps):
         w.launch(i)
     e1.record()
-    torch.cuda.synchronize()
+    while not e1.query():     # the end of the region is seen by polling: a blocking wait wakes up tens of microseconds late
+        pass
     wall = time.perf_counter() - t0
+    torch.cuda.synchronize()
     region_us = e0.elapsed_time(e1) * 1e3 / steps
     # single launches: one event pair around each (adds the cost of the two event records)
     n = min(steps, 200)
@@ -146,6 +196,74 @@ def time_gpu(w: Workload, steps: int, warmup: int):
     torch.cuda.synchronize()
     per = [a.elapsed_time(b) * 1e3 for a, b in ev]
     return wall, region_us, per
+
+
+def _event_time_us(fn, n: int) -> float:
+    for i in range(min(n, 200)):
+        fn(i)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(n):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / n
+
+
+def same_traffic_reference(w: 'Workload', steps: int):
+    """Kernels that move the same bytes as the configuration's operator and do no arithmetic to speak of, timed
+    on the same rotating buffers with HIP events:
+      * the library's own traffic-only kernel (tk_stream_floor: the operator's loads and stores, nothing else);
+      * a stock PyTorch elementwise kernel of the same byte shape (comparison of the input with zero, or of its two
+        halves, into a bool tensor of the output's shape);
+      * this entry point on four rows, replayed from a HIP graph of 100 launches: what one launch costs between
+        dependent launches in a stream, whatever its size.
+    They overwrite the output buffers; the caller runs the operator again before looking at results.
+    None where the configuration's traffic has no such stand-in (masked rows, half-byte codes)."""
+    if w.cfg not in (1, 2, 3):
+        return None
+    n = max(steps, 400)
+    outs = [o.view(torch.bool) for o in w.out]
+    rows, cols = w.x[0].shape[0], w.x[0].shape[1] // (2 if w.cfg == 3 else 1)
+    stream = w.main_stream
+
+    def stock(i):
+        x = w.x[i % w.nsets]
+        if w.cfg == 3:
+            torch.gt(x[:, :cols], x[:, cols:], out=outs[i % w.nsets])
+        else:
+            torch.gt(x, 0, out=outs[i % w.nsets])
+
+    def floor(i):
+        k = i % w.nsets
+        rc = w.lib.tk_stream_floor(w.x[k].data_ptr(), rows, cols, 1 if w.cfg == 3 else 0, w.out[k].data_ptr(),
+                                   0 if w.cfg == 2 else w.sf[k].data_ptr(), stream)
+        if rc != 0:
+            raise RuntimeError(f'tk_stream_floor failed with status {rc}')
+
+    res = {}
+    us = _event_time_us(floor, n)
+    res['traffic_only_kernel'] = {'what': 'tk_stream_floor: the loads and stores of this operator, no arithmetic',
+                                  'us_per_call': round(us, 3), 'pct_of_hbm_peak': round(w.bytes / us / 1e3 / HBM_PEAK_GBS * 100, 2)}
+    us = _event_time_us(stock, n)
+    moved = w.bytes - (0 if w.cfg == 2 else w.sf[0].numel() * w.sf[0].element_size())      # the stock kernel writes no scales
+    res['stock_torch_kernel'] = {'what': 'torch.gt into a bool tensor of the output shape (same bytes per element, no scales)',
+                                 'us_per_call': round(us, 3), 'pct_of_hbm_peak': round(moved / us / 1e3 / HBM_PEAK_GBS * 100, 2)}
+    # launch cost: 100 launches on four rows in one graph, so that the host's enqueue rate does not limit it
+    small = w.small_launch
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        small(side.cuda_stream)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(100):
+                small(side.cuda_stream)
+    torch.cuda.synchronize()
+    us = _event_time_us(lambda i: graph.replay(), 20) / 100
+    res['launch_cost_us'] = round(us, 3)
+    res['launch_cost_what'] = 'this entry point on four rows (128 for the per-block cast), per launch, 100 launches per HIP graph replay'
+    return res
 
 
 def time_two_streams(w: Workload, steps: int):
@@ -174,12 +292,16 @@ def copy_calibration(n_copies: int = 20, mib: int = 256):
     return {'copy_calibration': {'copies': n_copies, 'bytes_read_each': mib << 20, 'bytes_written_each': mib << 20}}
 
 
-def cpu_baseline(w: Workload, budget_s: float = 12.0):
+def cpu_baseline(w: Workload, budget_s: float = 12.0, min_runs: int = 3):
     """Times the CPU oracle on the full workload (repeated until the budget is used) and checks the
     GPU result of buffer set 0 against it."""
     from oracle import torch_ref
     from tests._util import dense_bytes, fp8_code_report
-    threads = min(16, os.cpu_count() or 1)
+    # threads: the CPUs this process may run on (the affinity mask and OMP_NUM_THREADS, which the GPU boxes set to
+    # their per-GPU share of the host); host_cores: what the machine has
+    host_cores = os.cpu_count() or 1
+    share = len(os.sched_getaffinity(0)) if hasattr(os, 'sched_getaffinity') else host_cores
+    threads = max(1, min(share, int(os.environ.get('OMP_NUM_THREADS', share) or share)))
     torch.set_num_threads(threads)
     d = w.host
     x = d['x']
@@ -198,12 +320,13 @@ def cpu_baseline(w: Workload, budget_s: float = 12.0):
     ref = run()   # warm-up, and the parity reference
     times = []
     t_start = time.perf_counter()
-    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 200):
+    while len(times) < min_runs or (time.perf_counter() - t_start < budget_s and len(times) < 200):
         t0 = time.perf_counter()
         run()
         times.append(time.perf_counter() - t0)
     med = statistics.median(times)
 
+    w.launch(0)        # other legs of the benchmark may have written to the output buffers since
     codes, sf = w.result(0)
     torch.cuda.synchronize()
     frac, one_step = fp8_code_report(dense_bytes(codes.cpu()), dense_bytes(ref[0])) if w.cfg != 5 else \
@@ -215,14 +338,16 @@ def cpu_baseline(w: Workload, budget_s: float = 12.0):
     else:
         sf_rel = float((a != b).float().mean())
     parity = {'codes_differing_frac': frac, 'code_diffs_one_step': one_step, 'scale_max_rel_err': sf_rel}
-    base = {'value': round(w.bytes / med / 1e9, 3), 'unit': 'GB/s', 'cores': threads, 'kind': 'port',
+    base = {'value': round(w.bytes / med / 1e9, 3), 'unit': 'GB/s', 'cores': threads, 'host_cores': host_cores, 'kind': 'port',
             'ms_per_call': round(med * 1e3, 3),
             'sample': f'full workload, {len(times)} timed calls of the torch CPU oracle after 1 warm-up (median)'}
     return base, parity
 
 
-def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_streams: bool = True):
+def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_streams: bool = True, preheat_ms: float = 40.0,
+                 cpu_budget_s: float = 12.0, with_reference: bool = True):
     w = Workload(cfg)
+    heated = preheat(w, preheat_ms)
     wall, kern_us, per = time_gpu(w, steps, warmup)
     ms_per_step = wall / steps * 1e3
     value = w.bytes / (wall / steps) / 1e9
@@ -234,35 +359,58 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_str
         'dtype': 'f32', 'data': 'synthetic',
         'config': {'workload': WORKLOADS[cfg], 'algorithmic_bytes': w.bytes, 'buffer_sets': w.nsets,
                    'boundary': 'C ABI (ctypes), preallocated outputs'},
+        'preheat_ms': round(heated, 1),
         'us_per_call': round(ms_per_step * 1e3, 3), 'pct_of_hbm_peak': round(100 * value / HBM_PEAK_GBS, 2),
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
                      'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': MEASURED_TRAFFIC_BYTES[cfg],
                      'kernel_us': round(kern_us, 3), 'timing': f'HIP events around the {steps} timed launches / {steps}',
                      'single_launch_us_median': round(statistics.median(per), 3), 'single_launch_us_min': round(min(per), 3)},
     }
+    if with_reference:
+        ref = same_traffic_reference(w, steps)
+        if ref is not None:
+            line['same_traffic_reference'] = ref
     # informational: what the same entry point sustains when independent calls overlap
     if with_two_streams:
-        us2 = time_two_streams(w, steps)
+        us2 = time_two_streams(w, max(steps, 200))
         line['two_streams'] = {'us_per_call': round(us2, 3), 'GBps': round(w.bytes / us2 / 1e3, 1),
                                'pct_of_hbm_peak': round(w.bytes / us2 / 1e3 / HBM_PEAK_GBS * 100, 2),
                                'note': 'calls alternate over two HIP streams; not used for value'}
     if with_cpu:
-        line['cpu_baseline'], line['parity'] = cpu_baseline(w)
+        line['cpu_baseline'], line['parity'] = cpu_baseline(w, cpu_budget_s, 3 if cpu_budget_s >= 6 else 1)
     return line
+
+
+def short_form(line: dict, cfg: int) -> dict:
+    """One entry of the `configs` array."""
+    out = {'cfg': cfg, 'workload': line['config']['workload'], 'us': line['roofline']['kernel_us'],
+           'us_wall': line['us_per_call'], 'GBps': line['roofline']['achieved'], 'frac': line['roofline']['frac']}
+    if 'cpu_baseline' in line:
+        out['cpu_ms'] = line['cpu_baseline']['ms_per_call']
+        out['parity'] = line['parity']
+    if 'same_traffic_reference' in line:
+        ref = line['same_traffic_reference']
+        out['traffic_only_kernel_us'] = ref['traffic_only_kernel']['us_per_call']
+        out['stock_torch_kernel_us'] = ref['stock_torch_kernel']['us_per_call']
+        out['launch_cost_us'] = ref['launch_cost_us']
+    return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=5000)
-    ap.add_argument('--warmup', type=int, default=2000,
-                    help='untimed launches first; the GPU needs ~15 ms of load to reach its steady clocks')
+    ap.add_argument('--warmup', type=int, default=2000, help='untimed launches directly before the timed ones')
+    ap.add_argument('--preheat-ms', type=float, default=40.0,
+                    help='untimed launches for this many milliseconds before the warm-up: the GPU needs ~15 ms of load to '
+                         'reach its steady clocks')
     ap.add_argument('--config', type=int, default=3, choices=sorted(WORKLOADS))
-    ap.add_argument('--all-configs', action='store_true', help='also print one line per other configuration to stderr')
+    ap.add_argument('--only', action='store_true', help='leave out the `configs` array (the other four configurations)')
+    ap.add_argument('--all-configs', action='store_true', help='also print the full line of every other configuration to stderr')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU-oracle baseline / parity leg')
     ap.add_argument('--single-stream-only', action='store_true',
-                    help='skip the informational two-stream leg (for kernel traces: overlapping launches there would '
-                         'inflate the per-kernel durations)')
+                    help='skip the informational two-stream leg and the same-traffic reference kernel (for kernel traces: '
+                         'overlapping launches there would inflate the per-kernel durations)')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run plain device copies of known size (reference kernel for hardware-counter runs)')
     args = ap.parse_args()
@@ -271,12 +419,20 @@ def main():
                  'run one process per GPU on its own row range). Use --gpus 1.')
     if not torch.cuda.is_available():
         sys.exit('bench.py needs a GPU')
-    if args.all_configs:
+    two = not args.single_stream_only
+    line = bench_config(args.config, args.steps, args.warmup, not args.no_cpu, two, args.preheat_ms, 12.0, two)
+    if not args.only:
+        # the other configurations with the same steps and warm-up, a short CPU leg each (one timed call of the oracle
+        # after its warm-up call, which is also the parity reference)
+        others = []
         for cfg in sorted(WORKLOADS):
-            if cfg != args.config:
-                print(json.dumps(bench_config(cfg, args.steps, args.warmup, not args.no_cpu, not args.single_stream_only)),
-                      file=sys.stderr, flush=True)
-    line = bench_config(args.config, args.steps, args.warmup, not args.no_cpu, not args.single_stream_only)
+            if cfg == args.config:
+                continue
+            full = bench_config(cfg, args.steps, args.warmup, not args.no_cpu, False, args.preheat_ms, 0.0, two)
+            if args.all_configs:
+                print(json.dumps(full), file=sys.stderr, flush=True)
+            others.append(short_form(full, cfg))
+        line['configs'] = others
     if args.copy_calibration:
         line.update(copy_calibration())
     print(json.dumps(line), flush=True)

@@ -320,6 +320,16 @@ int tk_check_expand_to_fused(const void *x, int64_t num_tokens, int64_t row_byte
                              const void *x_sf, int sf_cols, const void *out_sf, int64_t out_sf_ld, int sf_col_major);
 
 /* Text for a tk_status value (or "hip error" for positive codes). Never NULL. */
+/*
+ * tk_stream_floor: measurement aid with no counterpart in the reference.  A kernel with the memory traffic of the
+ * cast kernels (the same streaming 16-byte loads of a bf16 matrix, one byte written per element with the same
+ * write-through 8-byte stores, one 4-byte word per 128 columns if sf != NULL) and no arithmetic; with two_halves the
+ * input has 2 * cols columns and both halves are read per output element, as by tk_swiglu_per_token_cast.  bench.py
+ * times it beside the real operators: what it takes is what the access pattern costs on the machine.
+ *   requirements cols % 1024 == 0; x 16-byte, out 8-byte aligned
+ */
+int tk_stream_floor(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, void *stream);
+
 const char *tk_strerror(int status);
 /* TK_QUANT_VERSION the library was built from. */
 int tk_version(void);

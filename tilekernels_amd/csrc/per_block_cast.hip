@@ -1,9 +1,9 @@
 // Per-block (bm x bk, bm/bk in {32, 128}) block-scaled cast to E4M3 / E2M1 for gfx950.
 //
-// A workgroup of 512 threads owns one 128 x 128 tile, i.e. 1, 4 or 16 scale blocks.  Thread
-// (t, c) = (tid / 16, tid % 16) holds the 8 elements at columns 8c.. of rows t, t+32, t+64, t+96:
-// four 16-byte streaming loads per thread (bf16), all issued up front; the tile stays in registers
-// between the amax reduction and the conversion, so HBM is read once.  The amax of a block is
+// A workgroup owns one tile of 128 rows x TW columns (TW = 128 with 512 threads, or 512 with 1024 threads: see the
+// table at the launch code), i.e. 1 to 64 scale blocks.  With TW = 128, thread (t, c) = (tid / 16, tid % 16) holds
+// the 8 elements at columns 8c.. of rows t, t+32, t+64, t+96: four 16-byte streaming loads per thread (bf16), all
+// issued up front; the tile stays in registers between the amax reduction and the conversion, so HBM is read once.  The amax of a block is
 // reduced over the bk/8 lanes that share it with DPP, then across row slots and waves through one
 // LDS exchange (a partial per 16-lane row, one barrier, vector reads).
 //
@@ -34,13 +34,15 @@ struct PerBlockParams {
 #define TK_PB_LAUNCH_ARGS(p) \
     (p).x, (p).out, (p).sf.base, (p).sf.ld, (p).M, (p).K, (p).tiles_m, (p).tiles_k, (p).round_sf, (p).mode, (p).sf.layout, (p).sf.nm, (p).sf.nk
 
-// THREADS: 256 or 512 threads per tile (8 or 4 rows per thread).
+// TW: columns of a tile (128, 256 or 512); a tile is 128 rows x TW columns.
+// THREADS: threads per tile.
 // FULL: the tile lies wholly inside the matrix, so no bounds checks are compiled in.
-template <typename InT, int FMT, int BM, int BK, int THREADS, bool FULL>
+template <typename InT, int FMT, int BM, int BK, int TW, int THREADS, bool FULL>
 __device__ __forceinline__ void per_block_cast_tile(const PerBlockParams &p) {
-    constexpr int SUBM = kBlockTile / BM, SUBK = kBlockTile / BK;   // scale blocks per tile
+    constexpr int LPR = TW / 8;                                      // lanes along a row of the tile
+    constexpr int SUBM = kBlockTile / BM, SUBK = TW / BK;            // scale blocks per tile
     constexpr int LPG = BK / 8;                                      // lanes sharing a block in one row
-    constexpr int TR = THREADS / 16;                                 // rows covered by one pass of the workgroup
+    constexpr int TR = THREADS / LPR;                                // rows covered by one pass of the workgroup
     constexpr int NI = kBlockTile / TR;                              // rows per thread
     constexpr int IPB = BM / TR;                                     // of which per scale block
     static_assert(IPB >= 1, "a pass of the workgroup must not span two scale blocks");
@@ -49,8 +51,8 @@ __device__ __forceinline__ void per_block_cast_tile(const PerBlockParams &p) {
 
     const int tile_m = blockIdx.y, tile_k = blockIdx.x;   // 2-D grid: no division on the way to the first load
 
-    const int t = threadIdx.x >> 4, c = threadIdx.x & 15;
-    const int col = tile_k * kBlockTile + c * 8;
+    const int t = threadIdx.x / LPR, c = threadIdx.x % LPR;
+    const int col = tile_k * TW + c * 8;
     const int bj = (c * 8) / BK;
     const bool col_ok = FULL || col < p.K;
     const int row0 = tile_m * kBlockTile + t;
@@ -121,30 +123,48 @@ __device__ __forceinline__ void per_block_cast_tile(const PerBlockParams &p) {
 // FULL_GRID: M and K are multiples of 128.  Otherwise only the tiles on the lower and right edges take the
 // bounds-checked path; the choice is uniform over the workgroup.  (With every tile checked, bf16 [32767, 4096] took
 // 63.9 us against 59.1 us for [32768, 4096].)
-template <typename InT, int FMT, int BM, int BK, int THREADS, bool FULL_GRID>
+template <typename InT, int FMT, int BM, int BK, int TW, int THREADS, bool FULL_GRID>
 __global__ __launch_bounds__(THREADS) void per_block_cast_kernel(TK_PB_KERNEL_ARGS) {
     TK_PB_KERNEL_UNPACK;
     if constexpr (FULL_GRID) {
-        per_block_cast_tile<InT, FMT, BM, BK, THREADS, true>(p);
+        per_block_cast_tile<InT, FMT, BM, BK, TW, THREADS, true>(p);
     } else {
-        if (((int)blockIdx.y + 1) * kBlockTile <= p.M && ((int)blockIdx.x + 1) * kBlockTile <= p.K)
-            per_block_cast_tile<InT, FMT, BM, BK, THREADS, true>(p);
+        if (((int)blockIdx.y + 1) * kBlockTile <= p.M && ((int)blockIdx.x + 1) * TW <= p.K)
+            per_block_cast_tile<InT, FMT, BM, BK, TW, THREADS, true>(p);
         else
-            per_block_cast_tile<InT, FMT, BM, BK, THREADS, false>(p);
+            per_block_cast_tile<InT, FMT, BM, BK, TW, THREADS, false>(p);
     }
 }
 
-// 512 threads per 128 x 128 tile (4 rows per thread).  Measured on MI355X at bf16 [7168, 2048] ->
-// E4M3 128x128: 9.2 us per call, against 9.4 us with 256 threads (8 rows per thread) and 9.8 us with 1024 (2 rows).
-constexpr int kPerBlockThreads = 512;
+// Tile shapes, measured on MI355X for bf16 -> E4M3 128x128 (us per call):
+//                                          [2048,2048]  [7168,2048]  [4096,4096]  [4096,7168]  [8192,4096]  [16384,7168]
+//   128 x 128, 512 threads (4 rows/thread)     4.07         9.13        10.02        15.58        17.46        52.1
+//   128 x 512, 1024 threads (8 rows/thread)    6.02         8.60         9.19        16.36        18.45
+//   128 x 512, 512 threads (16 rows/thread)    6.31         8.87         9.82        16.59        20.37        58.8
+//   128 x 256, 1024 threads                    4.72         9.30        10.57        16.39        18.06
+// (128 x 128 with 256 threads: 9.4 at [7168,2048], with 1024: 9.8.)  A wave of a 512-column tile reads 1 KB of one
+// row per load instruction instead of 256 bytes of four rows, which pays while the matrix has too few 128 x 128
+// tiles to fill the GPU several times over (here 896 and 1024 tiles: 3.5 and 4 workgroups per CU) and costs where it
+// has many, or so few that whole CUs would stay empty.  The wide tile is used for bf16 input inside that window.
+constexpr int kPerBlockThreads = 512, kWideTile = 512, kWideThreads = 1024;
+constexpr int64_t kWideMinTiles = 512, kWideMaxTiles = 1280;     // in 128 x 128 tiles
+
+template <typename InT, int FMT, int BM, int BK, int TW, int THREADS>
+static void launch_per_block_3(const PerBlockParams &p, hipStream_t stream) {
+    const dim3 grid((unsigned)((p.K + TW - 1) / TW), (unsigned)p.tiles_m), block(THREADS);
+    if (p.M % kBlockTile == 0 && p.K % TW == 0)
+        hipLaunchKernelGGL((per_block_cast_kernel<InT, FMT, BM, BK, TW, THREADS, true>), grid, block, 0, stream, TK_PB_LAUNCH_ARGS(p));
+    else
+        hipLaunchKernelGGL((per_block_cast_kernel<InT, FMT, BM, BK, TW, THREADS, false>), grid, block, 0, stream, TK_PB_LAUNCH_ARGS(p));
+}
 
 template <typename InT, int FMT, int BM, int BK>
 static void launch_per_block_2(const PerBlockParams &p, hipStream_t stream) {
-    const dim3 grid((unsigned)p.tiles_k, (unsigned)p.tiles_m), block(kPerBlockThreads);
-    if (p.M % kBlockTile == 0 && p.K % kBlockTile == 0)
-        hipLaunchKernelGGL((per_block_cast_kernel<InT, FMT, BM, BK, kPerBlockThreads, true>), grid, block, 0, stream, TK_PB_LAUNCH_ARGS(p));
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_k;
+    if (sizeof(InT) == 2 && p.K % kWideTile == 0 && tiles >= kWideMinTiles && tiles <= kWideMaxTiles)
+        launch_per_block_3<InT, FMT, BM, BK, kWideTile, kWideThreads>(p, stream);
     else
-        hipLaunchKernelGGL((per_block_cast_kernel<InT, FMT, BM, BK, kPerBlockThreads, false>), grid, block, 0, stream, TK_PB_LAUNCH_ARGS(p));
+        launch_per_block_3<InT, FMT, BM, BK, kBlockTile, kPerBlockThreads>(p, stream);
 }
 
 template <typename InT, int FMT>

@@ -1,0 +1,70 @@
+// Measurement aid: a kernel with the memory traffic of the cast kernels and no arithmetic.
+//
+// A wave takes PIECES consecutive 512-column pieces of one row of a bf16 matrix, all its 16-byte loads issued
+// before the first is used (the same streaming loads as the casts), and writes one byte per element (the same
+// 8-byte write-through stores), plus one 4-byte word per 128 columns where the operator it stands beside writes
+// scales.  With `two_halves` the row has 2 * cols elements and a lane reads the piece of both halves, as the fused
+// SwiGLU cast does.  The bytes stored are the XOR of the words loaded, so no load can be dropped by the compiler;
+// there is no reduction, no conversion, no cross-lane step.  What this kernel takes on a given shape is what the
+// access pattern costs on the machine; the difference to the real operator is the operator's arithmetic.
+#include "tk_device.hpp"
+#include "tk_host.hpp"
+
+namespace tk {
+
+template <int PIECES, bool TWO>
+__global__ __launch_bounds__(kThreads) void stream_floor_kernel(const bf16_t *x, int rows, int cols, uint8_t *out, uint32_t *sf,
+                                                                int tiles_k) {
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const int tile_m = tile_grid_row(tiles_k == 1), tile_k = tile_grid_col(tiles_k == 1);
+    const int row = tile_m * kWaves + wave;
+    if (row >= rows) return;
+    const int col = tile_k * PIECES * kStripCols + lane * 8;
+    const int64_t ld = (int64_t)cols * (TWO ? 2 : 1);
+    const bf16_t *src = x + row * ld + col;
+    u32x4 a[PIECES], b[PIECES];
+#pragma unroll
+    for (int r = 0; r < PIECES; ++r) {
+        a[r] = ld_stream16(src + r * kStripCols);
+        b[r] = TWO ? ld_stream16(src + cols + r * kStripCols) : u32x4{0u, 0u, 0u, 0u};
+    }
+    uint32_t fold = 0;
+#pragma unroll
+    for (int r = 0; r < PIECES; ++r) {
+        const u32x4 v = a[r] ^ b[r];
+        st_stream8(out + (int64_t)row * cols + col + r * kStripCols, u32x2{v.x ^ v.z, v.y ^ v.w});
+        fold ^= v.x;
+    }
+    // one word per 128-column group: 4 per piece, the wave's PIECES * 4 words are one contiguous run
+    if (sf != nullptr && (lane & 15) < PIECES)
+        st_stream4(sf + (int64_t)row * (cols / 128) + (tile_k * PIECES + (lane & 15)) * 4 + (lane >> 4), fold);
+}
+
+}  // namespace tk
+
+using namespace tk;
+
+extern "C" int tk_stream_floor(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, void *stream) {
+    if (rows < 0 || cols <= 0 || cols % 1024 != 0) return TK_ERR_BAD_SHAPE;
+    if (rows > INT32_MAX - 64 || cols > (INT32_MAX - 1024) / 2) return TK_ERR_TOO_LARGE;
+    if (rows == 0) return TK_OK;
+    if (!x || !out) return TK_ERR_NULL_POINTER;
+    if (!aligned_to(x, 16) || !aligned_to(out, 8) || !aligned_to(sf, 4)) return TK_ERR_MISALIGNED;
+    const int pieces = cols % 2048 == 0 ? 4 : 2;
+    const int tiles_k = (int)(cols / (pieces * kStripCols)), tiles_m = (int)((rows + kWaves - 1) / kWaves);
+    const dim3 grid = tile_grid(tiles_k, tiles_m);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bf16_t *xp = static_cast<const bf16_t *>(x);
+    uint8_t *op = static_cast<uint8_t *>(out);
+    uint32_t *sp = static_cast<uint32_t *>(sf);
+#define TK_FLOOR_LAUNCH(P, T) hipLaunchKernelGGL((stream_floor_kernel<P, T>), grid, dim3(kThreads), 0, s, xp, (int)rows, (int)cols, op, sp, tiles_k)
+    if (pieces == 4) {
+        if (two_halves) TK_FLOOR_LAUNCH(4, true);
+        else TK_FLOOR_LAUNCH(4, false);
+    } else {
+        if (two_halves) TK_FLOOR_LAUNCH(2, true);
+        else TK_FLOOR_LAUNCH(2, false);
+    }
+#undef TK_FLOOR_LAUNCH
+    return (int)hipGetLastError();
+}

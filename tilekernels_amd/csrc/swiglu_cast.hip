@@ -13,11 +13,6 @@
 #include "tk_device.hpp"
 #include "tk_host.hpp"
 
-// Hook for timeline instrumentation in experiments; expands to nothing in the library.
-#ifndef TK_TRACE
-#define TK_TRACE(point)
-#endif
-
 namespace tk {
 
 struct SwigluParams {
@@ -137,7 +132,6 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
         const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * (2 * (int64_t)p.H) + col;
         constexpr int kRowStep = ROW ? 0 : 1, kColStep = ROW ? kStripCols : 0;
 
-        TK_TRACE(0);
         Raw8<InT> rg[RPW], ru[RPW];
         bool live[RPW];   // wave-uniform
         // the mask entries of all rows are fetched before the first of them is looked at: one scalar
@@ -168,7 +162,6 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
             }
         }
 
-        TK_TRACE(1);
         // dead rows hold zeros, so they flow through as v = 0 and only their scale is overridden
         float v[RPW][8], amax[RPW];
 #pragma unroll
@@ -227,7 +220,6 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
         for (int r = 0; r < RPW; ++r)
             if ((FULL || col + r * kColStep < p.H) && (FULL || row0 + r * kRowStep < p.R))
                 quantise_store8<TK_E4M3, false>(v[r], rs.inv[r], p.out + (int64_t)(row0 + r * kRowStep) * p.H, col + r * kColStep);
-        TK_TRACE(2);
         if constexpr (!DIRECT) {
             __syncthreads();
             if (ROWC) sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);

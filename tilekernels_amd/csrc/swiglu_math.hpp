@@ -11,17 +11,18 @@ namespace tk {
 // the exp: 1 + e is one IEEE addition, the quotient is corrected to (almost always) the IEEE
 // quotient, and the products that follow are single roundings in the reference's order.
 //
-// exp(-g) = 2^(g * -log2 e).  Rounding that product would put |g|*2^-24 of absolute error into the
-// exponent, so the constant is split into hi + lo and the lo part is applied to first order:
-// 2^(g*hi + g*lo) = 2^(g*hi) * (1 + g*lo*ln 2).
-//   bf16 input: hi keeps 15 significant bits, so g*hi is exact for an 8-bit significand
-//   fp32 input: the rounding error of g*hi is recovered with an fma and joins the lo term
+// exp(-g) = 2^(g * -log2 e) on v_exp_f32.
+//   bf16 input: one product with float(-log2 e).  Its rounding puts up to |g| * 1.44 * 2^-24 of absolute error into
+//               the exponent, i.e. a relative error of |g| * 6e-8 in exp(-g); that only reaches the result where
+//               exp(-g) dominates 1 + exp(-g) (gates below about -3), whose outputs are small against the group
+//               maximum that sets the scale.  Against the CPU evaluation at bf16 [8192, 4096], N(0,1): 4.2e-7 of the
+//               codes differ (budget 1e-4), each by one step, scales within 3.1e-7 (budget 1e-6); a hi/lo split of
+//               the constant (two more operations per element) brought the codes to 2.4e-7 and cost 0.08 us of 14.6.
+//   fp32 input: the constant is split into hi + lo and the rounding error of g*hi is recovered with an fma, both
+//               applied to first order: 2^(g*hi + t) = 2^(g*hi) * (1 + t * ln 2).
 // The gate is capped at -88 inside the exponential only (the CPU's exp overflows to inf at -88.7 and
 // its quotient becomes -0): e and 1 + e then stay finite, the reciprocal underflows and the corrected
 // quotient is -0 or a value below 1e-36, never inf * 0.
-#ifndef TK_SWIGLU_NEWTON
-#define TK_SWIGLU_NEWTON 1
-#endif
 
 // max(g, -88) on the bit pattern: negative floats order like their patterns as unsigned integers, and
 // every non-negative float has a smaller pattern than -88, so one integer min does it.  (A float max
@@ -35,11 +36,7 @@ __device__ __forceinline__ float floor_at_minus_88(float g) {
 template <typename InT> __device__ __forceinline__ float exp_neg(float g);
 
 template <> __device__ __forceinline__ float exp_neg<bf16_t>(float g) {
-    constexpr float nh = -1.44268798828125f;             // -log2(e) cut to 15 significant bits (0xBFB8AA00)
-    constexpr float nl_ln2 = -4.8884952e-06f;            // (-log2(e) - nh) * ln 2
-    const float gc = floor_at_minus_88(g);
-    const float e0 = __builtin_amdgcn_exp2f(gc * nh);    // exact product
-    return __builtin_fmaf(e0, gc * nl_ln2, e0);
+    return __builtin_amdgcn_exp2f(floor_at_minus_88(g) * -1.4426950408889634f);
 }
 
 template <> __device__ __forceinline__ float exp_neg<float>(float g) {
@@ -52,14 +49,12 @@ template <> __device__ __forceinline__ float exp_neg<float>(float g) {
     return __builtin_fmaf(e0, tl * 0.6931471805599453f, e0);
 }
 
-// g / d from r ~ 1/d: one Newton step on the quotient (two fmas)
+// g / d from r ~ 1/d: one Newton step on the quotient (two fmas).  Without the step the quotient is off by an ulp
+// often enough to matter where many elements share one value: with the gate clamped to 0.5 every clamped element sits
+// on the same rounding boundary, and 1.0e-4 of the codes then differed from the CPU's (the whole budget).
 __device__ __forceinline__ float quotient_with(float g, float d, float r) {
     const float q0 = g * r;
-#if TK_SWIGLU_NEWTON
     return __builtin_fmaf(__builtin_fmaf(-d, q0, g), r, q0);
-#else
-    return q0;
-#endif
 }
 __device__ __forceinline__ float quotient(float g, float d) { return quotient_with(g, d, __builtin_amdgcn_rcpf(d)); }
 
