@@ -159,6 +159,13 @@ def _format_sf(sf_bits: torch.Tensor, col_major: bool, packed: bool) -> torch.Te
       col-major : fp32 [nm, nk], strides (1, round_up(nm, 4))
       packed    : int32 [nm, ceil(nk/4)], strides (1, round_up(nm, 4)); byte t of word [m, j] is the
                   biased exponent of group 4j+t, zero beyond nk
+
+    One deliberate deviation from the torch statement this file restates: for a single column (nk == 1, or one
+    packed word) tile_kernels/torch/cast.py:216 returns strides (1, 1), because ``.T.contiguous().T`` of a
+    one-column tensor keeps row-major strides, while the reference's kernel path returns a transposed view of its
+    ``[nk, round_up(nm, 4)]`` storage, i.e. (1, round_up(nm, 4)) (tile_kernels/quant/common.py:141-165, 186-193).
+    This function returns the kernel path's strides for every nk, so that one rule describes the layout; values
+    and shape are the same either way, and the reference's tests flatten both sides before they compare.
     """
     nm, nk = sf_bits.shape
     if not col_major:

@@ -115,6 +115,23 @@ def test_scale_layouts(M, K, blk):
     assert (a - x.float()).abs().max() <= x.float().abs().max() * 2 ** -3
 
 
+@pytest.mark.parametrize('packed', [False, True])
+@pytest.mark.parametrize('M', [1, 6, 37])
+def test_single_column_of_column_major_scales_keeps_the_kernel_path_strides(M, packed):
+    """One block along the row: the scale tensor is [M, 1] with strides (1, round_up(M, 4)), as the reference's kernel
+    path returns it (a transposed view of [1, round_up(M, 4)] storage), not the (1, 1) that its torch statement's
+    `.T.contiguous().T` leaves for a single column."""
+    x = torch.randn((M, 128)).to(torch.bfloat16)
+    _, sf = torch_ref.cast(x, 'e4m3', (1, 128), round_sf=True, use_tma_aligned_col_major_sf=True, use_packed_ue8m0=packed)
+    assert tuple(sf.shape) == (M, 1) and sf.stride() == (1, (M + 3) // 4 * 4)
+    assert sf.dtype == (torch.int32 if packed else torch.float32)
+    _, row = torch_ref.cast(x, 'e4m3', (1, 128), round_sf=True)
+    if packed:
+        assert torch.equal(sf.flatten() & 0xFF, (row.view(torch.int32).flatten() >> 23))
+    else:
+        assert torch.equal(sf.flatten(), row.flatten())
+
+
 def test_empty_input_shapes():
     x = torch.empty((0, 256), dtype=torch.bfloat16)
     c, s = torch_ref.cast(x, 'e4m3', (1, 128))

@@ -67,6 +67,8 @@ template <typename T> __device__ __forceinline__ const void *elem_ptr(const void
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+// the same three words at an address that is only 4-byte aligned (the 12-byte E5M6 pieces): the plain type claims 16
+typedef u32x3 u32x3_a4 __attribute__((aligned(4)));
 
 // one_col: the grid is a single column of tiles (wave-uniform)
 __device__ __forceinline__ int tile_grid_row(bool one_col) { return (int)(one_col ? blockIdx.x : (blockIdx.z << kGridRowsLog2) + blockIdx.y); }
@@ -203,7 +205,7 @@ __device__ __forceinline__ float e5m6_value(uint32_t top12_in_bits_15_4) {
 template <> struct Raw8<e5m6in_t> {
     u32x3 w;
     float s;
-    __device__ __forceinline__ void load(const void *p) { w = __builtin_nontemporal_load(reinterpret_cast<const u32x3 *>(p)); }
+    __device__ __forceinline__ void load(const void *p) { w = __builtin_nontemporal_load(reinterpret_cast<const u32x3_a4 *>(p)); }
     __device__ __forceinline__ void load(const void *p, bool ok) {
         w = u32x3{0u, 0u, 0u};
         if (ok) load(p);
@@ -421,7 +423,7 @@ __device__ __forceinline__ void quantise_store8(const float (&v)[8], float inv, 
     for (int i = 0; i < 8; ++i) q[i] = v[i] * inv;
     if (FMT == TK_E4M3) st_stream8(out_row + col, pack_e4m3x8<CLAMP>(q));
     else if (FMT == TK_E2M1) st_stream4(out_row + (col >> 1), pack_e2m1x8(q));
-    else __builtin_nontemporal_store(pack_e5m6x8(q), reinterpret_cast<u32x3 *>(out_row + (col >> 3) * 12));
+    else __builtin_nontemporal_store(pack_e5m6x8(q), reinterpret_cast<u32x3_a4 *>(out_row + (col >> 3) * 12));
 }
 
 // ---------------------------------------------------------------------------------------------
