@@ -367,7 +367,11 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_str
                      'single_launch_us_median': round(statistics.median(per), 3), 'single_launch_us_min': round(min(per), 3)},
     }
     if with_reference:
-        ref = same_traffic_reference(w, steps)
+        try:        # a side measurement: its failure must not cost the line
+            ref = same_traffic_reference(w, steps)
+        except Exception as e:      # noqa: BLE001
+            ref = {'error': f'{type(e).__name__}: {e}'}
+            torch.cuda.synchronize()
         if ref is not None:
             line['same_traffic_reference'] = ref
     # informational: what the same entry point sustains when independent calls overlap
@@ -388,7 +392,7 @@ def short_form(line: dict, cfg: int) -> dict:
     if 'cpu_baseline' in line:
         out['cpu_ms'] = line['cpu_baseline']['ms_per_call']
         out['parity'] = line['parity']
-    if 'same_traffic_reference' in line:
+    if 'same_traffic_reference' in line and 'error' not in line['same_traffic_reference']:
         ref = line['same_traffic_reference']
         out['traffic_only_kernel_us'] = ref['traffic_only_kernel']['us_per_call']
         out['stock_torch_kernel_us'] = ref['stock_torch_kernel']['us_per_call']
@@ -428,7 +432,11 @@ def main():
         for cfg in sorted(WORKLOADS):
             if cfg == args.config:
                 continue
-            full = bench_config(cfg, args.steps, args.warmup, not args.no_cpu, False, args.preheat_ms, 0.0, two)
+            try:
+                full = bench_config(cfg, args.steps, args.warmup, not args.no_cpu, False, args.preheat_ms, 0.0, two)
+            except Exception as e:      # noqa: BLE001  (the headline line is printed whatever happens to a side leg)
+                others.append({'cfg': cfg, 'workload': WORKLOADS[cfg], 'error': f'{type(e).__name__}: {e}'})
+                continue
             if args.all_configs:
                 print(json.dumps(full), file=sys.stderr, flush=True)
             others.append(short_form(full, cfg))
