@@ -176,10 +176,12 @@ def time_gpu(w: 'Workload', steps: int, warmup: int):
         w.launch(i)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
+    todo = [w.calls[i % w.nsets] for i in range(steps)]
     e0.record()          # torch's current stream is the stream the launches go to
-    for i in range(steps):
-        w.launch(i)
+    t0 = time.perf_counter()
+    for fn, call_args in todo:
+        if fn(*call_args) != 0:
+            raise RuntimeError('launch failed')
     e1.record()
     while not e1.query():     # the end of the region is seen by polling: a blocking wait wakes up tens of microseconds late
         pass
