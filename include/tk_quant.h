@@ -254,7 +254,8 @@ int tk_check_per_block_cast_lossless(const void *x, int64_t M, int64_t K, const 
  * any of the three layouts.
  * Stands behind tile_kernels.quant.cast_back and per_token_cast_back
  * (tile_kernels/quant/cast_back_kernel.py:77-143, cast_back_e5m6_kernel.py:12-41, 141-176).
- *   requirements K % 8 == 0, bk % 8 == 0; out 16-byte aligned; x 8-byte (E4M3) / 4-byte (E2M1, E5M6) aligned
+ *   requirements K % 8 == 0; bk 1, 2, 4 (per-channel scales) or a multiple of 8; out 16-byte aligned;
+ *                x 8-byte (E4M3) / 4-byte (E2M1, E5M6) aligned
  */
 int tk_cast_back(const void *x, int x_fmt, int64_t M, int64_t K, const void *x_sf, int64_t x_sf_ld, int x_sf_layout,
                  int bm, int bk, void *out, int out_dtype, void *stream);

@@ -239,6 +239,20 @@ def test_reduce_fused_validation(lib):
     assert check_rf(lib, T=0, pos=0, out=0, x=0) == OK
 
 
+def test_cast_back_validation(lib):
+    def check(x=P, fmt=0, M=64, K=1024, sf=P, ld=None, layout=0, bm=1, bk=128, out=P, dt=0):
+        ld = (-(-K // bk) if bk > 0 else K) if ld is None else ld
+        return lib.tk_check_cast_back(x, fmt, M, K, sf, ld, layout, bm, bk, out, dt)
+    assert check() == OK
+    assert check(bm=128, bk=1) == OK and check(bm=128, bk=2) == OK and check(bm=128, bk=4) == OK     # per-channel scales
+    assert check(bk=3) == GROUP and check(bk=12) == GROUP and check(bk=0) == GROUP and check(bm=0) == GROUP
+    assert check(bm=128, bk=1, ld=1000) == STRIDE                       # one scale per column: the row of scales is K long
+    assert check(K=1020) == SHAPE
+    assert check(fmt=7) == FMT and check(dt=5) == DTYPE
+    assert check(out=0) == NULLP and check(sf=0) == NULLP
+    assert check(M=0, x=0, sf=0, out=0) == OK
+
+
 def test_moe_layout_validation(lib):
     ws = lib.tk_fused_mapping_workspace_bytes(4096, 8, 256)
     assert ws > 0

@@ -163,6 +163,46 @@ __global__ __launch_bounds__(kThreads) void cast_back_flat_kernel(const void *x,
     }
 }
 
+// Scale blocks narrower than a lane's 8 codes (bk = 1, 2 or 4: per-channel scales, as tile_kernels.quant.cast_back is
+// called with x_block_size (128, 1)): every code of a piece has its own scale column, so a lane fetches 8 / bk scales
+// beside its codes.  Pieces are laid end to end as in the kernel above; a lane writes its own 8 values (fp32: two
+// 16-byte stores).
+template <typename InT, bool OUT_F32>
+__global__ __launch_bounds__(kThreads) void cast_back_fine_kernel(const void *x, void *out, void *a_sf, int64_t a_sf_ld, int M, int K, int ppr,
+                                                                  unsigned ppr_recip, int bm, int bk, int a_sf_layout, int nm, int nk) {
+    const SfRef sf{a_sf, a_sf_ld, a_sf_layout, nm, nk};
+    const unsigned total = (unsigned)M * (unsigned)ppr;
+    const unsigned piece = blockIdx.x * (unsigned)kThreads + threadIdx.x;
+    if (piece >= total) return;
+    unsigned q = __umulhi(piece, ppr_recip), rem = piece - q * (unsigned)ppr;
+    if (rem >= (unsigned)ppr) { ++q; rem -= (unsigned)ppr; }
+    const int row = (int)q, col = (int)rem * 8;
+    Raw8<InT> raw;
+    raw.load(elem_ptr<InT>(x, row, K, col));
+    raw.s = 1.0f;                       // exact: the one rounding is the product with the element's own scale below
+    const int mb = row / bm;
+    float sc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sc[i] = sf_load_select(sf, mb, (col + i) / bk);
+    float v[8];
+    raw.get(v);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = v[i] * sc[i];
+    const int64_t idx = (int64_t)row * K + col;
+    if constexpr (OUT_F32) {
+        u32x4 *dst = reinterpret_cast<u32x4 *>(reinterpret_cast<float *>(out) + idx);
+        __builtin_nontemporal_store(u32x4{f2u(v[0]), f2u(v[1]), f2u(v[2]), f2u(v[3])}, dst);
+        __builtin_nontemporal_store(u32x4{f2u(v[4]), f2u(v[5]), f2u(v[6]), f2u(v[7])}, dst + 1);
+    } else {
+        u32x4 w;
+        w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[0], v[1]}), bf16x2));
+        w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[2], v[3]}), bf16x2));
+        w.z = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[4], v[5]}), bf16x2));
+        w.w = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[6], v[7]}), bf16x2));
+        __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(out) + idx));
+    }
+}
+
 template <typename InT, bool OUT_F32, bool WIDE>
 static void launch_cast_back_2(const void *x, void *out, const void *sf, int64_t sf_ld, int M, int K, int sf_layout, int bm, int bk,
                                hipStream_t stream) {
@@ -199,6 +239,13 @@ static hipError_t launch_cast_back(const void *x, void *out, const void *sf, int
     // against 16.2 us): a 2-row tile then uses 8 bytes of each scale line it touches
     // rows that fill less than 80 % of their 512-column strips
     const int64_t strips = (K + kStripCols - 1) / kStripCols, pieces = (int64_t)M * (K / 8);
+    if (bk < 8) {
+        const int64_t blocks = (pieces + kThreads - 1) / kThreads;
+        hipLaunchKernelGGL((cast_back_fine_kernel<InT, OUT_F32>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, x, out,
+                           const_cast<void *>(sf), sf_ld, M, K, K / 8,
+                           (unsigned)(K == 8 ? 0xFFFFFFFFull : (1ull << 32) / (uint64_t)(K / 8)), bm, bk, sf_layout, (M + bm - 1) / bm, (K + bk - 1) / bk);
+        return hipGetLastError();
+    }
     if (K * 5 < strips * kStripCols * 4 && pieces < INT32_MAX - 4 * kThreads) {   // pieces are numbered in 32 bits
         const int64_t blocks = (pieces + 2 * kThreads - 1) / (2 * kThreads);
         hipLaunchKernelGGL((cast_back_flat_kernel<InT, OUT_F32>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, x, out,
@@ -223,7 +270,8 @@ extern "C" int tk_check_cast_back(const void *x, int x_fmt, int64_t M, int64_t K
     if (x_sf_layout < TK_SF_ROW_F32 || x_sf_layout > TK_SF_COL_UE8M0) return TK_ERR_BAD_LAYOUT;
     if (M < 0 || K <= 0 || K % 8 != 0) return TK_ERR_BAD_SHAPE;
     if (M > INT32_MAX - 64 || K > INT32_MAX - 1024) return TK_ERR_TOO_LARGE;
-    if (bm < 1 || bk < 8 || bk % 8 != 0) return TK_ERR_BAD_GROUP;
+    if (bm < 1 || bk < 1 || (bk < 8 ? 8 % bk != 0 : bk % 8 != 0)) return TK_ERR_BAD_GROUP;   // 1, 2, 4 or a multiple of 8 columns per scale
+    if (bk < 8 && M * (K / 8) > INT32_MAX - 4 * kThreads) return TK_ERR_TOO_LARGE;
     if (M == 0) return TK_OK;
     if (!x || !x_sf || !out) return TK_ERR_NULL_POINTER;
     if (!aligned_to(x, x_fmt == TK_E4M3 ? 8 : 4) || !aligned_to(out, 16)) return TK_ERR_MISALIGNED;   // E5M6: 12-byte pieces of 4-byte words
