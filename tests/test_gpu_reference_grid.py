@@ -4,7 +4,8 @@ after clear_unused_sf for the comparison, check_bias on the dequantised result, 
 (tests/quant/test_per_token_cast.py:51-166, test_per_block_cast.py:36-110,
 test_swiglu_forward_and_per_token_cast.py:34-140).  The reference runs the full product of its options; here the
 product is enumerated in the same order and every STRIDE-th combination is run, so that all values of all options
-occur and the CPU oracle, which is the slow side, stays within a couple of minutes (TK_FULL_TEST=1 runs them all).
+occur and the CPU oracle, which is the slow side, stays within a couple of minutes (TK_FULL_TEST=1 runs them all;
+TK_GRID_SHIFT=n moves every sample n combinations along, so that successive runs cover other parts of the product).
 """
 import os
 
@@ -16,6 +17,7 @@ from oracle import torch_ref
 pytestmark = pytest.mark.gpu
 
 FULL = os.getenv('TK_FULL_TEST') in ('1', 'true', 'True')
+SHIFT = int(os.getenv('TK_GRID_SHIFT', '0'))
 
 
 def _tk():
@@ -33,7 +35,7 @@ def _ids(params):
 
 
 def _sample(params, stride, offset=0):
-    return params if FULL else params[offset::stride]
+    return params if FULL else params[(offset + SHIFT) % stride::stride]
 
 
 def to_host(t: torch.Tensor) -> torch.Tensor:
