@@ -215,7 +215,8 @@ int tk_check_per_channel_cast(const void *x, int x_dtype, const float *x_sf, int
  * accumulated in fp32 with one fused multiply-add per term, k ascending; topk_weights, x_sf ([num_expanded]
  * fp32) and sf (one fp32 on the device) may each be NULL (factor 1).  x: bf16 or fp32 [num_expanded, hidden],
  * contiguous; out: the type of x, or E4M3 bytes with out_dtype = TK_OUT_E4M3.  Positions outside [0, num_expanded) are
- * skipped; with num_expanded == 0 (x may then be NULL) the result is zeros.
+ * skipped; with num_expanded == 0 (x may then be NULL) the result is zeros.  The E4M3 conversion does not saturate: a
+ * scaled sum beyond +-448 becomes NaN (0x7F / 0xFF), as torch's conversion in the reference's statement of the operator does.
  * Stands behind tile_kernels.moe.reduce_fused (tile_kernels/moe/reduce_fused_kernel.py:70-135; oracle
  * tile_kernels/torch/reduce_fused.py:14-72).
  *   requirements hidden % 8 == 0; x and out 16-byte (E4M3 out: 8-byte) aligned

@@ -55,3 +55,19 @@ def test_per_block_cast_lossless_after_the_gpu_fp4_cast():
     a = tk.quant.cast_back(w4, 'fp32', (1, 32))
     b = tk.quant.cast_back(w8, 'fp32', (128, 128))
     assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+
+
+def test_per_block_cast_lossless_with_exponents_far_apart():
+    """Input scales more than 127 binades apart inside one output block: the small values vanish (+-0), nothing wraps."""
+    tk = _tk()
+    g = torch.Generator().manual_seed(17)
+    rows, hidden = 256, 1024
+    codes = torch.randint(-128, 128, (rows, hidden // 2), generator=g, dtype=torch.int16).to(torch.int8)
+    biased = torch.tensor([1, 10, 100, 121, 122, 150, 249, 250], dtype=torch.int32)
+    e = biased[torch.randint(0, len(biased), (rows, hidden // 32), generator=g)]
+    sf = (e << 23).view(torch.float32)
+    for out_block in [(128, 128), (32, 32), (1, 128)]:
+        want = torch_ref.per_block_cast_lossless((codes, sf), 'e4m3', (1, 32), out_block, round_sf=True)
+        got = tk.quant.per_block_cast_lossless((codes.cuda(), sf.cuda()), 'e4m3', (1, 32), out_block, round_sf=True)
+        assert_same(got[0], want[0], 'codes')
+        assert_same(got[1], want[1], 'scales')

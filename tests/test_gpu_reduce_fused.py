@@ -75,3 +75,16 @@ def test_reduce_fused_without_any_live_position():
             got = tk.moe.reduce_fused(x.cuda(), torch.rand((5, 3)).cuda(), t2p.cuda(), fp8_format=fp8)
             want = torch_ref.reduce_fused(x, torch.rand((5, 3)), t2p, fp8_format=fp8)
             assert_same(got, want, f'{dtype} {fp8}')
+
+
+def test_reduce_fused_e4m3_output_beyond_the_format_range():
+    """Scaled sums beyond +-448 are not saturated: they become NaN codes, as in the oracle (torch's conversion)."""
+    tk = _tk()
+    x = torch.tensor([[300.0, -300.0, 100.0, 447.0, 465.0, -480.0, 1.0, 0.0]] * 2, dtype=torch.float32).repeat(1, 32)
+    t2p = torch.tensor([[0, 1]], dtype=torch.int32)
+    w = torch.ones((1, 2))
+    want = torch_ref.reduce_fused(x, w, t2p, 'e4m3')
+    got = tk.moe.reduce_fused(x.cuda(), w.cuda(), t2p.cuda(), 'e4m3')
+    assert_same(got, want, 'codes')
+    codes = want.view(torch.uint8)[0, :8].tolist()
+    assert codes[0] == 0x7F and codes[1] == 0xFF and codes[3] == 0x7F and codes[2] != 0x7F      # 600, -600, 894 -> NaN; 200 is finite

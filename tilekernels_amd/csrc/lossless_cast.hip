@@ -6,7 +6,7 @@
 // at most 6 binades up stays at or below 384 <= 448, and shifted down by at most 5 stays a normal E4M3 number, so
 // E4M3 holds it exactly as long as the input exponents of one output block differ by no more than 11.  Beyond that
 // the reference asserts (tile_kernels/quant/per_block_cast_lossless_kernel.py:126); here the small values are
-// rounded by the conversion like any other.
+// rounded by the conversion like any other (to +-0 once they are 127 or more binades below the output exponent).
 //
 // A workgroup of 512 threads owns a 128 x 256 tile (every supported output block divides 128 x 128): a lane takes 16
 // consecutive codes (8 bytes; 8 codes where a block is narrower than 16 columns) of rows r, r + 32, ..., 4 in all, each
@@ -100,9 +100,11 @@ __global__ __launch_bounds__(kLlThreads) void lossless_fp4_to_fp8_kernel(const u
         if (!(col_ok && row < M)) continue;
         const int top = blk_max[row_in_tile >> obm_sh][bk_idx];
         const int e_out = top >= 6 ? top - 6 : 0;
-        // 2^(e_in - e_out) as a float: biased exponent e_in - e_out + 127, which the reference lets wrap when the input
-        // exponents of a block are further apart than it supports
-        const float scale = u2f((uint32_t)(e_in[p] - e_out + 127) << 23);
+        // 2^(e_in - e_out) as a float: biased exponent e_in - e_out + 127.  Input exponents 127 or more below the
+        // output's give 0 (such values are far below the smallest E4M3 step and become +-0, as with any scale below
+        // 2^-126; the reference asserts that a block's exponents lie within its range instead)
+        const int biased = e_in[p] - e_out + 127;
+        const float scale = u2f((uint32_t)(biased > 0 ? biased : 0) << 23);
         if constexpr (CODES == 8) {
             Raw8<e2m1in_t> raw;
             raw.w = code[p];
