@@ -191,7 +191,8 @@ def _to_gpu_like(t: torch.Tensor) -> torch.Tensor:
 @pytest.mark.parametrize('fmt', ['e4m3', 'e2m1'])
 @pytest.mark.parametrize('in_fmt', ['e4m3', 'e2m1'])
 @pytest.mark.parametrize('x_block', [(128, 128), (32, 32), (1, 128), (1, 32)])
-@pytest.mark.parametrize('M,K,N', [(401, 7168, 128), (401, 7168, 32), (37, 576, 128), (37, 576, 32), (130, 2048, 64)])
+@pytest.mark.parametrize('M,K,N', [(401, 7168, 128), (401, 7168, 32), (37, 576, 128), (37, 576, 32), (130, 2048, 64), (131, 4096, 32),
+                                   (7, 6144, 128)])
 def test_per_token_cast_of_quantised_input(M, K, N, x_block, in_fmt, fmt, mode):
     """Input = (codes, scales) of an earlier cast, in every scale layout; same structure as the
     quantised-input cases of the reference's tests/quant/test_per_token_cast.py:25-36."""
@@ -203,6 +204,25 @@ def test_per_token_cast_of_quantised_input(M, K, N, x_block, in_fmt, fmt, mode):
     want_codes, want_sf = torch_ref.cast(q, fmt, (1, N), x_block_size=x_block, **kw)
     qg = (q[0].cuda(), _to_gpu_like(q[1]))
     codes, sf = tk.quant.per_token_cast(qg, fmt, N, x_block_size=x_block, **kw)
+    assert_same(codes, want_codes, 'codes')
+    assert_same(sf, want_sf, 'sf')
+
+
+@pytest.mark.parametrize('fmt,N', [('e2m1', 32), ('e4m3', 128), ('e4m3', 32), ('e2m1', 64)])
+@pytest.mark.parametrize('pad,shift', [(0, 0), (16, 0), (8, 0), (16, 8), (32, 16)])
+def test_per_token_cast_of_strided_e4m3_codes(pad, shift, fmt, N):
+    """E4M3 codes handed over as a view with a row stride of K + pad bytes starting `shift` bytes into the row: rows
+    that are 16-byte aligned take the kernel with one 16-byte load per lane, the others the 8-byte one."""
+    tk = _tk()
+    M, K = 67, 4096
+    x = torch.randn((M, K)).to(torch.bfloat16)
+    q = torch_ref.cast(x, 'e4m3', (1, 128), round_sf=True)
+    want_codes, want_sf = torch_ref.cast(q, fmt, (1, N), x_block_size=(1, 128), round_sf=True)
+    wide = torch.zeros((M, K + pad), dtype=torch.uint8, device='cuda')
+    view = wide[:, shift:shift + K].view(torch.float8_e4m3fn)
+    view.view(torch.uint8).copy_(q[0].view(torch.uint8).cuda())
+    assert view.stride(0) == K + pad and view.data_ptr() % 16 == shift % 16
+    codes, sf = tk.quant.per_token_cast((view, q[1].cuda()), fmt, N, x_block_size=(1, 128), round_sf=True)
     assert_same(codes, want_codes, 'codes')
     assert_same(sf, want_sf, 'sf')
 

@@ -11,6 +11,8 @@
 //
 // Reference semantics: tile_kernels/quant/per_token_cast_kernel.py:65-154 (plain-tensor branch),
 // tile_kernels/quant/common.py:196-244.
+#include <type_traits>
+
 #include "tk_device.hpp"
 #include "tk_host.hpp"
 
@@ -164,6 +166,71 @@ __global__ __launch_bounds__(TILE == T_WIDE ? 64 * kMaxWideWaves : kThreads) voi
             else if (p.sf.layout == TK_SF_ROW_F32) sf_store_tile_rowmajor<ROWS, SGPR>(p.sf, stage, GPS, tile_m * ROWS, tile_k * GPS);
             else sf_store_tile_colmajor<ROWS, SGPR>(p.sf, stage, tile_m * ROWS, tile_k * SGPR);
         }
+    }
+}
+
+// E4M3 input with block scales -> E2M1, row-major output scales, K a multiple of RPW * 1024: one row per wave, a lane
+// taking 16 consecutive codes (one 16-byte load) of each of its RPW pieces of 1024 columns and writing their 16
+// output codes with one 8-byte store.  With 8 codes per lane, as in the kernel above, a wave's load instruction
+// moves 512 bytes and its store 256.  Measured on MI355X, 1 x 128 -> E2M1 1 x 32 (us per call, 8 / 16 codes per
+// lane): [8192, 4096] 12.0 / 10.9, [32768, 4096] 39.7 / 36.2, [16384, 8192] 39.6 / 35.1; with 4 pieces per wave
+// instead of 2: 11.4, 35.3, 34.1.  (E4M3 output, whose stores are 8 bytes per lane already, did not gain: [32768, 4096]
+// 43.5 -> 44.6.)  A group of G columns lives in G / 16 neighbouring lanes; the 16 codes of a lane share one input
+// scale (input blocks are multiples of 16 columns wide here).  Waves share nothing: no LDS, no barrier.
+template <int G, int RPW, bool FULL_GRID>
+__global__ __launch_bounds__(kThreads) void per_token_cast_q16_kernel(TK_PT_KERNEL_ARGS) {
+    TK_PT_KERNEL_UNPACK;
+    constexpr int kWide = 1024;                  // columns per piece
+    constexpr int LPG = G / 16, GPS = kWide / G;
+    constexpr int FMT = TK_E2M1;
+    using RS = RowScales<Fmt<FMT>::qmax, RPW, LPG>;
+    const bool one_col = RPW * kWide >= p.K;
+    const int tile_m = tile_grid_row(one_col), tile_k = tile_grid_col(one_col);
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const int strip = tile_k * RPW;
+    const int col = strip * kWide + lane * 16;
+    const int kgrp = strip * GPS + lane / LPG;
+    const int row0 = tile_m * kWaves + wave;
+    if constexpr (!FULL_GRID) {
+        if (row0 >= p.M) return;
+    }
+    Raw8<e4m3in_t> lo[RPW], hi[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+        const u32x4 w = ld_stream16(elem_ptr<e4m3in_t>(p.x, row0, p.x_ld, col + r * kWide));
+        lo[r].w = u32x2{w.x, w.y};
+        hi[r].w = u32x2{w.z, w.w};
+        lo[r].s = hi[r].s = sf_load(p.xsf, row0 / p.in_bm, (col + r * kWide) / p.in_bk);
+    }
+    float amax[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+        float a[8], b[8];
+        lo[r].get(a);
+        hi[r].get(b);
+        amax[r] = group_allmax<LPG>(__builtin_fmaxf(absmax8(a), absmax8(b)));
+    }
+    RS rs;
+    rs.compute(amax, Fmt<FMT>::floor_, p.round_sf != 0, lane);
+    // lane j (< A) of a group computed the scale of piece c*A + j; the wave's scales form one run of RPW * GPS floats
+    const int own = lane % LPG;
+    if (own < RS::A) {
+#pragma unroll
+        for (int c = 0; c < RS::NC; ++c)
+            st_stream4(reinterpret_cast<float *>(p.sf.base) + (int64_t)row0 * p.sf.ld + kgrp + (c * RS::A + own) * GPS, f2u(rs.own[c].sf));
+    }
+    uint8_t *out_row = p.out + (int64_t)row0 * (p.K / 2);
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+        float a[8], b[8];
+        lo[r].get(a);
+        hi[r].get(b);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            a[i] = a[i] * rs.inv[r];
+            b[i] = b[i] * rs.inv[r];
+        }
+        st_stream8(out_row + ((col + r * kWide) >> 1), u32x2{pack_e2m1x8(a), pack_e2m1x8(b)});
     }
 }
 
@@ -397,6 +464,19 @@ static void launch_per_token_group(PerTokenParams &p, hipStream_t stream) {
                                TK_PT_LAUNCH_ARGS(p));
             return;
             }
+        }
+    }
+    if constexpr (std::is_same<InT, e4m3in_t>::value && G >= 32 && FMT == TK_E2M1) {
+        constexpr int Q16_RPW = 2;
+        if (p.sf.layout == TK_SF_ROW_F32 && p.K % (Q16_RPW * 1024) == 0 && p.in_bk % 16 == 0 && aligned_to(p.x, 16) && p.x_ld % 16 == 0) {
+            const int tiles_m = (p.M + kWaves - 1) / kWaves, tiles_k = p.K / (Q16_RPW * 1024);
+            p.geom = tiles_k;
+            const dim3 grid = tile_grid(tiles_k, tiles_m);
+            if (p.M % kWaves == 0 && tile_grid_exact(tiles_k, tiles_m))
+                hipLaunchKernelGGL((per_token_cast_q16_kernel<G, Q16_RPW, true>), grid, dim3(kThreads), 0, stream, TK_PT_LAUNCH_ARGS(p));
+            else
+                hipLaunchKernelGGL((per_token_cast_q16_kernel<G, Q16_RPW, false>), grid, dim3(kThreads), 0, stream, TK_PT_LAUNCH_ARGS(p));
+            return;
         }
     }
     // Row-wise tiles where they fit the columns exactly.  Measured on MI355X against wide tiles: bf16 [4096, 7168] -> E4M3 14.85 ->
