@@ -194,3 +194,28 @@ def test_c_abi_combinations_the_wrappers_do_not_use(quantised, transpose):
     torch.cuda.synchronize()
     assert_same(out, want_codes, 'codes')
     assert_same(out_sf, want_sf, 'scales')
+
+
+@pytest.mark.parametrize('x_shift,out_shift', [(0, 0), (8, 0), (0, 8), (8, 8)])
+def test_fp8_input_with_buffers_that_are_only_8_byte_aligned(x_shift, out_shift):
+    """The FP8-input cast moves 16 bytes per lane where its buffers allow it and 8 bytes otherwise: both give the oracle's result."""
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    T, K = 272, 1152
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn((T, K), generator=g).to(torch.bfloat16)
+    xin = torch_ref.cast(x, 'e4m3', (1, 128))
+    want_codes, want_sf = torch_ref.per_channel_cast_fused(xin, 128, 128, True, None)
+    xbuf = torch.zeros(T * K + 16, dtype=torch.uint8, device='cuda')
+    xbuf[x_shift:x_shift + T * K].copy_(xin[0].view(torch.uint8).flatten().cuda())
+    obuf = torch.zeros(T * K + 16, dtype=torch.uint8, device='cuda')
+    sfd = xin[1].cuda()
+    out_sf = torch.empty(tuple(want_sf.shape), dtype=torch.float32, device='cuda')
+    rc = lib.tk_per_channel_cast(xbuf.data_ptr() + x_shift, 0, sfd.data_ptr(), T, K, None, T, obuf.data_ptr() + out_shift, out_sf.data_ptr(),
+                                 128, 1, 0, 0, 0, 0.0, _ffi.current_stream(obuf.device))
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    got = obuf[out_shift:out_shift + T * K].view(torch.float8_e4m3fn).reshape(T, K)
+    assert_same(got, want_codes, 'codes')
+    assert_same(out_sf, want_sf, 'scales')
+    assert int(obuf[:out_shift].sum()) == 0 and int(obuf[out_shift + T * K:].sum()) == 0
