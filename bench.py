@@ -19,6 +19,10 @@ of a stock PyTorch elementwise kernel that moves the same bytes (no arithmetic t
 buffers, next to the time per launch of this entry point on a four-row input (what a launch costs on
 this stack whatever its size).
 
+`roofline.traffic` is measured too: before it touches the GPU the script runs itself twice per configuration under
+rocprofv3 (FETCH_SIZE, then WRITE_SIZE, each scaled by a copy of known size in the same run; `--no-measure-traffic`
+skips this and reports the figures of earlier such runs).
+
 Before the `--warmup` launches the GPU is kept busy with the same launches for `--preheat-ms`
 milliseconds (untimed): its clocks need about 15 ms of load to settle, and a handful of 15 us
 launches does not provide that.
@@ -294,6 +298,80 @@ def copy_calibration(n_copies: int = 20, mib: int = 256):
     return {'copy_calibration': {'copies': n_copies, 'bytes_read_each': mib << 20, 'bytes_written_each': mib << 20}}
 
 
+def under_a_profiler() -> bool:
+    """Whether a ROCm profiler is loaded into this process.  Its tool library initialises the GPU before the program
+    starts, and a process in that state must not start other programs: the counter leg is skipped then.  (PyTorch
+    itself maps librocprofiler-register and libroctracer64; a profiler brings its tool library and its variables.)"""
+    env = os.environ
+    if env.get('HSA_TOOLS_LIB') or env.get('ROCP_TOOL_LIBRARIES') or any(k.startswith('ROCPROF') for k in env):
+        return True
+    if any(name in env.get('LD_PRELOAD', '') for name in ('rocprofiler-sdk', 'rocprofiler64', 'roctracer', 'rocprof-')):
+        return True
+    try:
+        with open('/proc/self/maps') as f:
+            return any('rocprofiler-sdk' in line or 'rocprofiler64' in line or 'tracer_tool' in line for line in f)
+    except OSError:
+        return True
+
+
+def measure_traffic(cfg: int, timeout_s: float = 60.0) -> dict:
+    """HBM bytes per launch of configuration `cfg`, from two hardware-counter runs of this script under rocprofv3
+    (FETCH_SIZE, then WRITE_SIZE: KiB per dispatch, one counter per run), each scaled by what the same counter reads
+    for the 256 MiB copies of --copy-calibration in the same run.  The profiler runs as a child process, so this
+    has to be called before the calling process touches the GPU."""
+    import collections
+    import csv
+    import glob
+    import shutil
+    import signal
+    import subprocess
+    import tempfile
+    exe = shutil.which('rocprofv3')
+    if exe is None:
+        raise RuntimeError('rocprofv3 is not on PATH')
+    tmp = tempfile.mkdtemp(prefix='tk_traffic_', dir='/tmp')
+    cal_bytes = 256 << 20
+    result = {}
+    try:
+        for counter in ('FETCH_SIZE', 'WRITE_SIZE'):
+            out_dir = os.path.join(tmp, counter)
+            cmd = [exe, '--pmc', counter, '--output-format', 'csv', '-d', out_dir, '-o', 'c', '--', sys.executable,
+                   os.path.abspath(__file__), '--only', '--no-cpu', '--single-stream-only', '--config', str(cfg), '--steps', '100',
+                   '--warmup', '20', '--preheat-ms', '0', '--copy-calibration', '--no-measure-traffic']
+            child = subprocess.Popen(cmd, cwd='/tmp', env=dict(os.environ, TMPDIR='/tmp'), stdout=subprocess.DEVNULL,
+                                     stderr=subprocess.DEVNULL, start_new_session=True)
+            try:
+                rc = child.wait(timeout_s)
+            except subprocess.TimeoutExpired:
+                os.killpg(child.pid, signal.SIGKILL)
+                child.wait()
+                raise RuntimeError(f'the {counter} run did not finish within {timeout_s:.0f} s')
+            if rc != 0:
+                raise RuntimeError(f'the {counter} run exited with {rc}')
+            files = glob.glob(os.path.join(out_dir, '**', '*counter_collection.csv'), recursive=True)
+            if not files:
+                raise RuntimeError(f'the {counter} run left no counter file')
+            per_kernel = collections.defaultdict(list)
+            with open(files[0], newline='') as f:
+                for row in csv.DictReader(f):
+                    if row['Counter_Name'] == counter:
+                        per_kernel[row['Kernel_Name']].append(float(row['Counter_Value']))
+            cal = [v for k, v in per_kernel.items() if 'CUDAFunctorOnSelf_add<int>' in k]
+            ours = [v for k, v in per_kernel.items() if 'tk::' in k and 'stream_floor' not in k]
+            if len(cal) != 1 or not ours:
+                raise RuntimeError(f'the {counter} run holds {len(cal)} calibration kernels and {len(ours)} kernels of the library')
+            mine = max(ours, key=len)                           # the timed kernel is the one with the most dispatches
+            scale = (cal_bytes / 1024.0) / (sum(cal[0]) / len(cal[0]))
+            result[counter] = {'kib_per_dispatch': round(sum(mine) / len(mine), 1), 'dispatches': len(mine), 'scale': round(scale, 5),
+                               'bytes': sum(mine) / len(mine) * scale * 1024.0}
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    return {'bytes': round(result['FETCH_SIZE']['bytes'] + result['WRITE_SIZE']['bytes']),
+            'read_bytes': round(result['FETCH_SIZE']['bytes']), 'written_bytes': round(result['WRITE_SIZE']['bytes']),
+            'fetch_scale': result['FETCH_SIZE']['scale'], 'write_scale': result['WRITE_SIZE']['scale'],
+            'dispatches': result['FETCH_SIZE']['dispatches']}
+
+
 def cpu_baseline(w: Workload, budget_s: float = 12.0, min_runs: int = 3):
     """Times the CPU oracle on the full workload (repeated until the budget is used) and checks the
     GPU result of buffer set 0 against it."""
@@ -347,7 +425,7 @@ def cpu_baseline(w: Workload, budget_s: float = 12.0, min_runs: int = 3):
 
 
 def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_streams: bool = True, preheat_ms: float = 40.0,
-                 cpu_budget_s: float = 12.0, with_reference: bool = True):
+                 cpu_budget_s: float = 12.0, with_reference: bool = True, traffic: dict = None):
     w = Workload(cfg)
     heated = preheat(w, preheat_ms)
     wall, kern_us, per = time_gpu(w, steps, warmup)
@@ -364,7 +442,10 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_str
         'preheat_ms': round(heated, 1),
         'us_per_call': round(ms_per_step * 1e3, 3), 'pct_of_hbm_peak': round(100 * value / HBM_PEAK_GBS, 2),
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': MEASURED_TRAFFIC_BYTES[cfg],
+                     'frac': round(achieved / HBM_PEAK_GBS, 4),
+                     'traffic': float(traffic['bytes']) if traffic and 'bytes' in traffic else MEASURED_TRAFFIC_BYTES[cfg],
+                     'traffic_source': ('rocprofv3 FETCH_SIZE and WRITE_SIZE runs started by this run' if traffic and 'bytes' in traffic
+                                        else 'earlier rocprofv3 counter runs of this script (profiles/)'),
                      'kernel_us': round(kern_us, 3), 'timing': f'HIP events around the {steps} timed launches / {steps}',
                      'single_launch_us_median': round(statistics.median(per), 3), 'single_launch_us_min': round(min(per), 3)},
     }
@@ -390,7 +471,8 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_str
 def short_form(line: dict, cfg: int) -> dict:
     """One entry of the `configs` array."""
     out = {'cfg': cfg, 'workload': line['config']['workload'], 'us': line['roofline']['kernel_us'],
-           'us_wall': line['us_per_call'], 'GBps': line['roofline']['achieved'], 'frac': line['roofline']['frac']}
+           'us_wall': line['us_per_call'], 'GBps': line['roofline']['achieved'], 'frac': line['roofline']['frac'],
+           'traffic': line['roofline']['traffic']}
     if 'cpu_baseline' in line:
         out['cpu_ms'] = line['cpu_baseline']['ms_per_call']
         out['parity'] = line['parity']
@@ -417,16 +499,30 @@ def main():
     ap.add_argument('--single-stream-only', action='store_true',
                     help='skip the informational two-stream leg and the same-traffic reference kernel (for kernel traces: '
                          'overlapping launches there would inflate the per-kernel durations)')
+    ap.add_argument('--no-measure-traffic', action='store_true',
+                    help='skip the hardware-counter leg: by default this script first runs itself twice per configuration under '
+                         'rocprofv3 (FETCH_SIZE, then WRITE_SIZE; a few seconds each) and reports the HBM bytes per launch measured '
+                         'there as roofline.traffic; without it, or if the profiler fails, the figures of earlier such runs are reported')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run plain device copies of known size (reference kernel for hardware-counter runs)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: this path has no multi-GPU component (rows are independent; '
                  'run one process per GPU on its own row range). Use --gpus 1.')
+    traffic = {}
+    if not args.no_measure_traffic and not under_a_profiler():        # child processes: started before this process touches the GPU
+        for cfg in ([args.config] if args.only else sorted(WORKLOADS)):
+            try:
+                traffic[cfg] = measure_traffic(cfg)
+            except Exception as e:      # noqa: BLE001  (a side measurement: the stored figure is reported instead)
+                traffic[cfg] = {'error': f'{type(e).__name__}: {e}'}
+                break                   # and the other configurations are not tried
     if not torch.cuda.is_available():
         sys.exit('bench.py needs a GPU')
     two = not args.single_stream_only
-    line = bench_config(args.config, args.steps, args.warmup, not args.no_cpu, two, args.preheat_ms, 12.0, two)
+    line = bench_config(args.config, args.steps, args.warmup, not args.no_cpu, two, args.preheat_ms, 12.0, two, traffic.get(args.config))
+    if traffic:
+        line['traffic_measurement'] = {str(c): t for c, t in traffic.items()}
     if not args.only:
         # the other configurations with the same steps and warm-up, a short CPU leg each (one timed call of the oracle
         # after its warm-up call, which is also the parity reference)
@@ -435,7 +531,7 @@ def main():
             if cfg == args.config:
                 continue
             try:
-                full = bench_config(cfg, args.steps, args.warmup, not args.no_cpu, False, args.preheat_ms, 0.0, two)
+                full = bench_config(cfg, args.steps, args.warmup, not args.no_cpu, False, args.preheat_ms, 0.0, two, traffic.get(cfg))
             except Exception as e:      # noqa: BLE001  (the headline line is printed whatever happens to a side leg)
                 others.append({'cfg': cfg, 'workload': WORKLOADS[cfg], 'error': f'{type(e).__name__}: {e}'})
                 continue
