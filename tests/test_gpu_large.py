@@ -133,6 +133,26 @@ def test_per_channel_cast_beyond_2g_elements(transpose):
         _same_bytes(sf[a // 128:b // 128], s_ref, f'sf[{a // 128}]')
 
 
+def test_casts_of_e4m3_codes_beyond_2g_elements():
+    """The two kernels that take E4M3 codes 16 to a lane: the re-quantisation to E2M1 and the per-channel cast."""
+    tk = _tk()
+    M, K = 282 * 128, 61440
+    assert M * K > LIMIT
+    x = _randn_bf16((M, K), 8)
+    q = tk.quant.per_token_cast(x, 'e4m3', 128, round_sf=True)
+    del x
+    codes4, sf4 = tk.quant.per_token_cast(q, 'e2m1', 32, x_block_size=(1, 128), round_sf=True)
+    codes8, sf8 = tk.quant.per_channel_cast_fused(q, 'e4m3', num_per_tokens=128, round_sf=True, num_per_channels=128)
+    for a, b in _windows(M, 128):
+        qw = (q[0][a:b].cpu(), q[1][a:b].cpu())
+        c_ref, s_ref = torch_ref.cast(qw, 'e2m1', (1, 32), x_block_size=(1, 128), round_sf=True)
+        _same_bytes(codes4[a:b], c_ref, f'e2m1 codes[{a}:{b}]')
+        _same_bytes(sf4[a:b], s_ref, f'e2m1 sf[{a}:{b}]')
+        c_ref, s_ref = torch_ref.per_channel_cast_fused(qw, 128, 128, True, None)
+        _same_bytes(codes8[a:b], c_ref, f'per-channel codes[{a}:{b}]')
+        _same_bytes(sf8[a // 128:b // 128], s_ref, f'per-channel sf[{a // 128}]')
+
+
 def test_expand_to_fused_beyond_4_gib():
     tk = _tk()
     T, K, E, hidden = 36000, 8, 64, 8192
