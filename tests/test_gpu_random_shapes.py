@@ -1,6 +1,7 @@
 """Seeded random shapes and options against the CPU oracle, to the same bars as the hand-picked cases: row counts,
 row lengths, formats, scale layouts, masks and weights are drawn at random so that the tile shape, the bounds handling
 and the scale layout of a call vary together.  Every seed collects its failing cases and fails once at the end."""
+import os
 import random
 
 import pytest
@@ -19,11 +20,15 @@ def _tk():
     return tilekernels_amd
 
 
+# TK_FUZZ_SEEDS=101,102,... adds runs with other seeds to the committed ones
+EXTRA_SEEDS = [int(v) for v in os.getenv('TK_FUZZ_SEEDS', '').split(',') if v.strip()]
+
+
 def _modes(rng):
     return rng.choice([(False, False, False), (False, True, False), (True, False, False), (True, True, False), (True, True, True)])
 
 
-@pytest.mark.parametrize('seed', [11, 12])
+@pytest.mark.parametrize('seed', [11, 12] + EXTRA_SEEDS)
 def test_random_casts_swiglu_and_moe_rows(seed):
     """per_token_cast, cast_back, per_block_cast, the fused SwiGLU cast, expand_to_fused and reduce_fused."""
     tk = _tk()
@@ -110,7 +115,7 @@ def test_random_casts_swiglu_and_moe_rows(seed):
     assert not failures, '\n'.join(failures)
 
 
-@pytest.mark.parametrize('seed', [21, 22])
+@pytest.mark.parametrize('seed', [21, 22] + EXTRA_SEEDS)
 def test_random_operators_around_the_path(seed):
     """The fused backward, the per-channel family, E5M6, the lossless re-blocking, the mapping, expansion with scales
     and re-quantisation of quantised input."""
