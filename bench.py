@@ -272,6 +272,69 @@ def same_traffic_reference(w: 'Workload', steps: int):
     return res
 
 
+def launch_timeline(cfg: int, launches: int = 14, preheat_ms: float = 40.0) -> dict:
+    """How a launch of the configuration's size is spent, from per-wave time stamps of the traffic-only kernel
+    (tk_stream_floor_timeline: the operator's loads and stores, every wave reporting its start, the arrival of its last
+    load, the issue and the acknowledgement of its stores on the 100 MHz real-time counter, and where it ran).
+    `launches` calls go out back to back on the rotating buffers; the first two are left out of the summary.
+    All times in microseconds; figures are means over the launches unless they say otherwise."""
+    import numpy as np
+    if cfg not in (1, 3):
+        raise SystemExit('--timeline knows the row-wise traffic of configurations 1 and 3')
+    w = Workload(cfg)
+    preheat(w, preheat_ms)
+    rows, cols = w.x[0].shape[0], w.x[0].shape[1] // (2 if cfg == 3 else 1)
+    words = int(w.lib.tk_stream_floor_stamp_words(rows, cols))
+    stamps = torch.zeros((launches, words), dtype=torch.int64, device=w.x[0].device)
+    torch.cuda.synchronize()
+    for i in range(launches):
+        k = i % w.nsets
+        rc = w.lib.tk_stream_floor_timeline(w.x[k].data_ptr(), rows, cols, 1 if cfg == 3 else 0, w.out[k].data_ptr(), w.sf[k].data_ptr(),
+                                            stamps[i].data_ptr(), w.main_stream)
+        if rc != 0:
+            raise RuntimeError(f'tk_stream_floor_timeline failed with status {rc}')
+    torch.cuda.synchronize()
+    t = stamps.cpu().numpy().reshape(launches, -1, 6)
+    tick = 0.01                                     # 100 MHz
+    bytes_per_wave = w.bytes / t.shape[1]
+    spans, gaps, ramp50, ramp99, first_data, med_data, xcd_start, xcd_end, mid_rate, tail10 = [], [], [], [], [], [], [], [], [], []
+    for i in range(2, launches):
+        a = t[i]
+        start = a[:, 0].min()
+        rel = (a[:, :4] - start) * tick
+        end = rel[:, 3].max()
+        spans.append(end)
+        if i + 1 < launches:
+            gaps.append((t[i + 1][:, 0].min() - a[:, 3].max()) * tick)
+        ramp50.append(float(np.percentile(rel[:, 0], 50)))
+        ramp99.append(float(np.percentile(rel[:, 0], 99)))
+        wait = rel[:, 1] - rel[:, 0]
+        first_data.append(float(wait.min()))
+        med_data.append(float(np.median(wait)))
+        xcc = a[:, 5] & 0xF
+        xcd_start.append([float(rel[xcc == x, 0].mean()) for x in range(8)])
+        xcd_end.append([float(rel[xcc == x, 3].max()) for x in range(8)])
+        mid = (rel[:, 1] >= 0.3 * end) & (rel[:, 1] < 0.7 * end)
+        mid_rate.append(float(mid.sum() * bytes_per_wave / (0.4 * end) / 1e3))       # GB/s of the operator's bytes
+        tail10.append(float(end - np.percentile(rel[:, 1], 90)))
+    mean = lambda v: round(float(np.mean(v)), 3)
+    xs, xe = np.array(xcd_start), np.array(xcd_end)
+    return {
+        'timeline': f'tk_stream_floor_timeline on the buffers of config {cfg}, {launches - 2} back-to-back launches',
+        'waves_per_launch': int(t.shape[1]),
+        'first_wave_to_last_acknowledgement_us': {'mean': mean(spans), 'min': round(min(spans), 3), 'max': round(max(spans), 3)},
+        'last_acknowledgement_to_first_wave_of_next_launch_us': {'mean': mean(gaps), 'min': round(min(gaps), 3), 'max': round(max(gaps), 3)},
+        'half_of_the_waves_started_after_us': mean(ramp50), 'all_but_1_percent_started_after_us': mean(ramp99),
+        'wave_start_to_its_last_load_us': {'shortest': mean(first_data), 'median': mean(med_data)},
+        'mean_wave_start_per_xcd_us': [round(float(v), 3) for v in xs.mean(axis=0)],
+        'last_acknowledgement_per_xcd_us': {'mean': [round(float(v), 3) for v in xe.mean(axis=0)],
+                                             'spread_within_a_launch_mean': mean(xe.max(axis=1) - xe.min(axis=1)),
+                                             'spread_within_a_launch_max': round(float((xe.max(axis=1) - xe.min(axis=1)).max()), 3)},
+        'operator_bytes_per_second_in_the_middle_40_percent_GBps': mean(mid_rate),
+        'last_tenth_of_the_loads_arrives_within_us_of_the_end': mean(tail10),
+    }
+
+
 def time_two_streams(w: Workload, steps: int):
     """Same calls, alternating over two streams: consecutive calls are independent batches, so the
     ramp-up of one overlaps the drain of the other.  Returns microseconds per call."""
@@ -503,12 +566,20 @@ def main():
                     help='skip the hardware-counter leg: by default this script first runs itself twice per configuration under '
                          'rocprofv3 (FETCH_SIZE, then WRITE_SIZE; a few seconds each) and reports the HBM bytes per launch measured '
                          'there as roofline.traffic; without it, or if the profiler fails, the figures of earlier such runs are reported')
+    ap.add_argument('--timeline', action='store_true',
+                    help='instead of the benchmark, print how a launch of the configuration\'s size is spent (per-wave time stamps '
+                         'of the traffic-only kernel over a few back-to-back launches; configurations 1 and 3)')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run plain device copies of known size (reference kernel for hardware-counter runs)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: this path has no multi-GPU component (rows are independent; '
                  'run one process per GPU on its own row range). Use --gpus 1.')
+    if args.timeline:
+        if not torch.cuda.is_available():
+            sys.exit('bench.py needs a GPU')
+        print(json.dumps(launch_timeline(args.config, preheat_ms=args.preheat_ms)), flush=True)
+        return
     traffic = {}
     if not args.no_measure_traffic and not under_a_profiler():        # child processes: started before this process touches the GPU
         for cfg in ([args.config] if args.only else sorted(WORKLOADS)):

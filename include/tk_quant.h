@@ -332,6 +332,18 @@ int tk_check_expand_to_fused(const void *x, int64_t num_tokens, int64_t row_byte
  */
 int tk_stream_floor(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, void *stream);
 
+/*
+ * tk_stream_floor_timeline: the same kernel reporting where and when each of its waves ran (no counterpart in the
+ * reference; bench.py --timeline reads it).  stamps receives tk_stream_floor_stamp_words(rows, cols) 64-bit words, six
+ * per wave in row order: the 100 MHz real-time counter at the wave's start, when its last load has arrived (this variant
+ * waits for all loads before its first store), when its stores are issued and when they are acknowledged, then the
+ * HW_ID and XCC_ID hardware registers.
+ *   requirements as tk_stream_floor; stamps 8-byte aligned
+ */
+int tk_stream_floor_timeline(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, void *stamps,
+                             void *stream);
+int64_t tk_stream_floor_stamp_words(int64_t rows, int64_t cols);
+
 const char *tk_strerror(int status);
 /* TK_QUANT_VERSION the library was built from. */
 int tk_version(void);

@@ -37,3 +37,28 @@ def test_stream_floor_rejects_bad_shapes():
     assert lib.tk_stream_floor(p, 4, 1000, 0, p, 0, None) != 0          # columns not a multiple of 1024
     assert lib.tk_stream_floor(0, 4, 1024, 0, p, 0, None) != 0          # null input
     assert lib.tk_stream_floor(0, 0, 1024, 0, 0, 0, None) == 0          # no rows: nothing to do
+
+
+@pytest.mark.parametrize('rows,cols,two', [(37, 2048, True), (64, 4096, False), (9, 3072, True)])
+def test_stream_floor_timeline_stamps_every_wave(rows, cols, two):
+    """The time-stamped variant writes the same output and, per wave, four non-decreasing times and its place."""
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    width = cols * (2 if two else 1)
+    xd = torch.randint(-2 ** 15, 2 ** 15, (rows, width), dtype=torch.int16, device='cuda')
+    stream = torch.cuda.current_stream().cuda_stream
+    out = [torch.zeros((rows, cols), dtype=torch.uint8, device='cuda') for _ in range(2)]
+    sf = [torch.zeros((rows, cols // 128), dtype=torch.int32, device='cuda') for _ in range(2)]
+    words = lib.tk_stream_floor_stamp_words(rows, cols)
+    assert words == rows * (cols // (2048 if cols % 2048 == 0 else 1024)) * 6
+    stamps = torch.zeros(words, dtype=torch.int64, device='cuda')
+    assert lib.tk_stream_floor(xd.data_ptr(), rows, cols, int(two), out[0].data_ptr(), sf[0].data_ptr(), stream) == 0
+    assert lib.tk_stream_floor_timeline(xd.data_ptr(), rows, cols, int(two), out[1].data_ptr(), sf[1].data_ptr(), stamps.data_ptr(), stream) == 0
+    assert lib.tk_stream_floor_timeline(xd.data_ptr(), rows, cols, int(two), out[1].data_ptr(), sf[1].data_ptr(), 0, stream) != 0     # no stamp buffer
+    torch.cuda.synchronize()
+    assert torch.equal(out[0], out[1]) and torch.equal(sf[0], sf[1])
+    t = stamps.cpu().numpy().reshape(-1, 6)
+    assert (t[:, 0] > 0).all()
+    assert (t[:, 0] <= t[:, 1]).all() and (t[:, 1] <= t[:, 2]).all() and (t[:, 2] <= t[:, 3]).all()
+    assert ((t[:, 3] - t[:, 0]) < 100 * 1000).all()             # well under a millisecond at 100 MHz
+    assert ((t[:, 5] & 0xF) < 8).all()                          # XCD number

@@ -7,14 +7,24 @@
 // SwiGLU cast does.  The bytes stored are the XOR of the words loaded, so no load can be dropped by the compiler;
 // there is no reduction, no conversion, no cross-lane step.  What this kernel takes on a given shape is what the
 // access pattern costs on the machine; the difference to the real operator is the operator's arithmetic.
+//
+// With STAMP every wave also reports when it ran: the 100 MHz real-time counter at its start, when its last load
+// has arrived (this variant waits for all loads before its first store), when its stores are issued and when they
+// are acknowledged, plus the hardware id registers that say where it ran (XCD, shader engine, CU, SIMD).  From these
+// stamps of a few back-to-back launches one reads how a launch of this size is spent: the gap between two launches, how
+// long the waves take to start, when the first data arrives, how evenly the XCDs finish.
 #include "tk_device.hpp"
 #include "tk_host.hpp"
 
 namespace tk {
 
-template <int PIECES, bool TWO>
+constexpr int kStampWords = 6;     // per wave: start, loads done, stores issued, stores acknowledged, HW_ID, XCC_ID
+
+template <int PIECES, bool TWO, bool STAMP>
 __global__ __launch_bounds__(kThreads) void stream_floor_kernel(const bf16_t *x, int rows, int cols, uint8_t *out, uint32_t *sf,
-                                                                int tiles_k) {
+                                                                int tiles_k, unsigned long long *stamps) {
+    unsigned long long t_start = 0, t_loaded = 0;
+    if constexpr (STAMP) t_start = wall_clock64();
     const int lane = threadIdx.x & 63, wave = wave_id();
     const int tile_m = tile_grid_row(tiles_k == 1), tile_k = tile_grid_col(tiles_k == 1);
     const int row = tile_m * kWaves + wave;
@@ -28,6 +38,10 @@ __global__ __launch_bounds__(kThreads) void stream_floor_kernel(const bf16_t *x,
         a[r] = ld_stream16(src + r * kStripCols);
         b[r] = TWO ? ld_stream16(src + cols + r * kStripCols) : u32x4{0u, 0u, 0u, 0u};
     }
+    if constexpr (STAMP) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        t_loaded = wall_clock64();
+    }
     uint32_t fold = 0;
 #pragma unroll
     for (int r = 0; r < PIECES; ++r) {
@@ -38,18 +52,33 @@ __global__ __launch_bounds__(kThreads) void stream_floor_kernel(const bf16_t *x,
     // one word per 128-column group: 4 per piece, the wave's PIECES * 4 words are one contiguous run
     if (sf != nullptr && (lane & 15) < PIECES)
         st_stream4(sf + (int64_t)row * (cols / 128) + (tile_k * PIECES + (lane & 15)) * 4 + (lane >> 4), fold);
+    if constexpr (STAMP) {
+        const unsigned long long t_issued = wall_clock64();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const unsigned long long t_acked = wall_clock64();
+        if (lane == 0) {
+            unsigned long long *q = stamps + ((int64_t)row * tiles_k + tile_k) * kStampWords;
+            q[0] = t_start;
+            q[1] = t_loaded;
+            q[2] = t_issued;
+            q[3] = t_acked;
+            q[4] = __builtin_amdgcn_s_getreg(63492);     // hwreg(HW_ID): wave, SIMD, CU, shader array and engine
+            q[5] = __builtin_amdgcn_s_getreg(63508);     // hwreg(XCC_ID)
+        }
+    }
 }
 
 }  // namespace tk
 
 using namespace tk;
 
-extern "C" int tk_stream_floor(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, void *stream) {
+static int stream_floor_launch(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, void *stamps,
+                               bool stamp, void *stream) {
     if (rows < 0 || cols <= 0 || cols % 1024 != 0) return TK_ERR_BAD_SHAPE;
     if (rows > INT32_MAX - 64 || cols > (INT32_MAX - 1024) / 2) return TK_ERR_TOO_LARGE;
     if (rows == 0) return TK_OK;
-    if (!x || !out) return TK_ERR_NULL_POINTER;
-    if (!aligned_to(x, 16) || !aligned_to(out, 8) || !aligned_to(sf, 4)) return TK_ERR_MISALIGNED;
+    if (!x || !out || (stamp && !stamps)) return TK_ERR_NULL_POINTER;
+    if (!aligned_to(x, 16) || !aligned_to(out, 8) || !aligned_to(sf, 4) || !aligned_to(stamps, 8)) return TK_ERR_MISALIGNED;
     const int pieces = cols % 2048 == 0 ? 4 : 2;
     const int tiles_k = (int)(cols / (pieces * kStripCols)), tiles_m = (int)((rows + kWaves - 1) / kWaves);
     const dim3 grid = tile_grid(tiles_k, tiles_m);
@@ -57,14 +86,37 @@ extern "C" int tk_stream_floor(const void *x, int64_t rows, int64_t cols, int tw
     const bf16_t *xp = static_cast<const bf16_t *>(x);
     uint8_t *op = static_cast<uint8_t *>(out);
     uint32_t *sp = static_cast<uint32_t *>(sf);
-#define TK_FLOOR_LAUNCH(P, T) hipLaunchKernelGGL((stream_floor_kernel<P, T>), grid, dim3(kThreads), 0, s, xp, (int)rows, (int)cols, op, sp, tiles_k)
+    unsigned long long *tp = static_cast<unsigned long long *>(stamps);
+#define TK_FLOOR_LAUNCH(P, T, S) \
+    hipLaunchKernelGGL((stream_floor_kernel<P, T, S>), grid, dim3(kThreads), 0, s, xp, (int)rows, (int)cols, op, sp, tiles_k, tp)
+#define TK_FLOOR_LAUNCH_2(P, T)          \
+    do {                                 \
+        if (stamp) TK_FLOOR_LAUNCH(P, T, true); \
+        else TK_FLOOR_LAUNCH(P, T, false);      \
+    } while (0)
     if (pieces == 4) {
-        if (two_halves) TK_FLOOR_LAUNCH(4, true);
-        else TK_FLOOR_LAUNCH(4, false);
+        if (two_halves) TK_FLOOR_LAUNCH_2(4, true);
+        else TK_FLOOR_LAUNCH_2(4, false);
     } else {
-        if (two_halves) TK_FLOOR_LAUNCH(2, true);
-        else TK_FLOOR_LAUNCH(2, false);
+        if (two_halves) TK_FLOOR_LAUNCH_2(2, true);
+        else TK_FLOOR_LAUNCH_2(2, false);
     }
+#undef TK_FLOOR_LAUNCH_2
 #undef TK_FLOOR_LAUNCH
     return (int)hipGetLastError();
+}
+
+extern "C" int tk_stream_floor(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, void *stream) {
+    return stream_floor_launch(x, rows, cols, two_halves, out, sf, nullptr, false, stream);
+}
+
+extern "C" int64_t tk_stream_floor_stamp_words(int64_t rows, int64_t cols) {
+    if (rows < 0 || cols <= 0 || cols % 1024 != 0) return 0;
+    const int pieces = cols % 2048 == 0 ? 4 : 2;
+    return rows * (cols / (pieces * kStripCols)) * kStampWords;
+}
+
+extern "C" int tk_stream_floor_timeline(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf,
+                                        void *stamps, void *stream) {
+    return stream_floor_launch(x, rows, cols, two_halves, out, sf, stamps, true, stream);
 }
