@@ -17,7 +17,9 @@ host cores for the same workload and doubles as the in-run parity check.  `confi
 figures, in short, for the other four benchmark configurations, and `same_traffic_reference` the time
 of a stock PyTorch elementwise kernel that moves the same bytes (no arithmetic to speak of) on the same
 buffers, next to the time per launch of this entry point on a four-row input (what a launch costs on
-this stack whatever its size).
+this stack whatever its size).  `launch_structure` says how a launch of this size is spent (gap between launches, start
+of the waves, first data, streaming rate, spread between the XCDs), from time stamps the traffic-only kernel takes per
+wave; `--timeline` prints only that.
 
 `roofline.traffic` is measured too: before it touches the GPU the script runs itself twice per configuration under
 rocprofv3 (FETCH_SIZE, then WRITE_SIZE, each scaled by a copy of known size in the same run; `--no-measure-traffic`
@@ -569,6 +571,8 @@ def main():
     ap.add_argument('--timeline', action='store_true',
                     help='instead of the benchmark, print how a launch of the configuration\'s size is spent (per-wave time stamps '
                          'of the traffic-only kernel over a few back-to-back launches; configurations 1 and 3)')
+    ap.add_argument('--no-launch-structure', action='store_true',
+                    help='leave out `launch_structure` (what --timeline prints, appended to the full line of configurations 1 and 3)')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run plain device copies of known size (reference kernel for hardware-counter runs)')
     args = ap.parse_args()
@@ -612,6 +616,11 @@ def main():
         line['configs'] = others
     if args.copy_calibration:
         line.update(copy_calibration())
+    if not args.only and not args.no_launch_structure and args.config in (1, 3):
+        try:        # a side measurement, taken after everything else: its failure must not cost the line
+            line['launch_structure'] = launch_timeline(args.config, preheat_ms=args.preheat_ms)
+        except Exception as e:      # noqa: BLE001
+            line['launch_structure'] = {'error': f'{type(e).__name__}: {e}'}
     print(json.dumps(line), flush=True)
 
 
