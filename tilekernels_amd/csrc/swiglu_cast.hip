@@ -423,10 +423,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KER
 // (T_ROW) instead of four rows: 14.75 -> 14.63.  fp32 input, whose pieces are twice the bytes (sixteen
 // 16-byte loads per lane with 4 pieces), is better off with 2: [16384, 2 x 2048] 59.5 -> 52.1 us,
 // [16384, 2 x 4096] 116.2 -> 98.2 us.
-#ifndef TK_SWIGLU_RPW
-#define TK_SWIGLU_RPW 4
-#endif
-template <typename InT> constexpr int swiglu_pieces() { return sizeof(InT) == 4 ? 2 : TK_SWIGLU_RPW; }
+template <typename InT> constexpr int swiglu_pieces() { return sizeof(InT) == 4 ? 2 : 4; }
 
 template <typename InT, int CLAMP, int RPW, int TILE>
 static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t stream) {
