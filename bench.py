@@ -337,6 +337,52 @@ def launch_timeline(cfg: int, launches: int = 14, preheat_ms: float = 40.0) -> d
     }
 
 
+VARIANTS = {'base': 0, 'pkfloor': 1, 'widest': 2, 'prio': 3, 'piecesf': 4, 'late': 5, 'ahead': 6, 'rounds': 7}
+
+
+def variant_ab(specs, steps: int, rounds: int = 4, preheat_ms: float = 40.0) -> dict:
+    """Times alternative structures of the headline kernel (tk_swiglu_cast_variant: measurement aids of the library, not
+    reachable from the Python API) against the product entry point on configuration 3's buffers: `rounds` rounds, each
+    timing the product and every variant in turn over `steps` launches with HIP events.  Every variant's codes and scales
+    are first compared with the product's, bit for bit.  `specs`: names from VARIANTS, each optionally followed by
+    ':<parameter>'."""
+    w = Workload(3)
+    preheat(w, preheat_ms)
+    x = w.host['x']
+    R, H = x.shape[0], x.shape[1] // 2
+    stream = w.main_stream
+    legs = [('product', lambda i: w.launch(i))]
+    for spec in specs:
+        name, _, par = spec.partition(':')
+        if name not in VARIANTS:
+            raise SystemExit(f'unknown variant {name!r}; known: {", ".join(VARIANTS)}')
+        code, param = VARIANTS[name], int(par) if par else 0
+
+        def call(i, code=code, param=param):
+            k = i % w.nsets
+            rc = w.lib.tk_swiglu_cast_variant(w.x[k].data_ptr(), R, H, w.out[k].data_ptr(), w.sf[k].data_ptr(), code, param, stream)
+            if rc != 0:
+                raise RuntimeError(f'tk_swiglu_cast_variant failed with status {rc}')
+        legs.append((spec, call))
+    w.launch(0)
+    torch.cuda.synchronize()
+    ref_codes, ref_sf = w.out[0].view(torch.uint8).clone(), w.sf[0].clone()
+    parity = {}
+    for spec, call in legs[1:]:
+        w.out[0].view(torch.uint8).fill_(0xAB)
+        w.sf[0].fill_(-1.0)
+        call(0)
+        torch.cuda.synchronize()
+        parity[spec] = bool(torch.equal(w.out[0].view(torch.uint8), ref_codes) and torch.equal(w.sf[0], ref_sf))
+    times = {spec: [] for spec, _ in legs}
+    for _ in range(rounds):
+        for spec, call in legs:
+            times[spec].append(round(_event_time_us(call, steps), 3))
+    return {'workload': WORKLOADS[3], 'steps': steps, 'rounds': rounds,
+            'us_per_launch': {k: {'median': round(statistics.median(v), 3), 'runs': v} for k, v in times.items()},
+            'identical_to_product': parity}
+
+
 def time_two_streams(w: Workload, steps: int):
     """Same calls, alternating over two streams: consecutive calls are independent batches, so the
     ramp-up of one overlaps the drain of the other.  Returns microseconds per call."""
@@ -573,6 +619,9 @@ def main():
                          'of the traffic-only kernel over a few back-to-back launches; configurations 1 and 3)')
     ap.add_argument('--no-launch-structure', action='store_true',
                     help='leave out `launch_structure` (what --timeline prints, appended to the full line of configurations 1 and 3)')
+    ap.add_argument('--variant', type=str, default=None,
+                    help='instead of the benchmark, time alternative structures of the headline kernel against the product: a comma-separated '
+                         f'list of {", ".join(VARIANTS)}, each optionally with ":<parameter>" (see csrc/swiglu_cast_variants.hip)')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run plain device copies of known size (reference kernel for hardware-counter runs)')
     args = ap.parse_args()
@@ -583,6 +632,11 @@ def main():
         if not torch.cuda.is_available():
             sys.exit('bench.py needs a GPU')
         print(json.dumps(launch_timeline(args.config, preheat_ms=args.preheat_ms)), flush=True)
+        return
+    if args.variant:
+        if not torch.cuda.is_available():
+            sys.exit('bench.py needs a GPU')
+        print(json.dumps(variant_ab(args.variant.split(','), min(args.steps, 4000), preheat_ms=args.preheat_ms)), flush=True)
         return
     traffic = {}
     if not args.no_measure_traffic and not under_a_profiler():        # child processes: started before this process touches the GPU

@@ -321,7 +321,6 @@ int tk_check_expand_to_fused(const void *x, int64_t num_tokens, int64_t row_byte
                              int num_topk, const int32_t *pos_to_expert, int64_t num_expanded, const void *out,
                              const void *x_sf, int sf_cols, const void *out_sf, int64_t out_sf_ld, int sf_col_major);
 
-/* Text for a tk_status value (or "hip error" for positive codes). Never NULL. */
 /*
  * tk_stream_floor: measurement aid with no counterpart in the reference.  A kernel with the memory traffic of the
  * cast kernels (the same streaming 16-byte loads of a bf16 matrix, one byte written per element with the same
@@ -344,6 +343,21 @@ int tk_stream_floor_timeline(const void *x, int64_t rows, int64_t cols, int two_
                              void *stream);
 int64_t tk_stream_floor_stamp_words(int64_t rows, int64_t cols);
 
+/*
+ * tk_swiglu_cast_variant: measurement aid with no counterpart in the reference.  Alternative structures of the kernel
+ * behind tk_swiglu_per_token_cast for its plain case (bf16 x[R, 2H], E4M3 codes, row-major fp32 1 x 128 scales, no mask,
+ * weights or clamp), each producing the same codes and scales bit for bit; bench.py --variant times them beside the
+ * product kernel, which is how the figures quoted for them can be measured again.  variant / param:
+ *   0 the product's structure (param: rows per workgroup 1, 2, 4 or 8; 0 = 4)      4 a scale division per piece and lane,
+ *   1 the gate's -88 cap on packed bf16 pairs (param as 0)                           each piece stored once converted
+ *   2 16-byte code stores after a lane-pair exchange (param as 0)                  5 variant 4 for waves whose first piece
+ *   3 wave priority raised once the first piece has arrived (param as 0)             arrives later than param * 10 ns
+ *   6 pieces requested param (1, 2) ahead instead of all at once                   7 param (1, 2) pieces per wave, not 4
+ *   requirements H % 2048 == 0, R % 8 == 0; x and out 16-byte aligned
+ */
+int tk_swiglu_cast_variant(const void *x, int64_t R, int64_t H, void *out, void *sf, int variant, int param, void *stream);
+
+/* Text for a tk_status value (or "hip error" for positive codes). Never NULL. */
 const char *tk_strerror(int status);
 /* TK_QUANT_VERSION the library was built from. */
 int tk_version(void);

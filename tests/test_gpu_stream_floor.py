@@ -27,7 +27,20 @@ def test_stream_floor_reads_and_writes_everything(rows, cols, two):
     q = w.reshape(rows, cols // 8, 4)
     want = np.stack([q[:, :, 0] ^ q[:, :, 2], q[:, :, 1] ^ q[:, :, 3]], axis=-1).reshape(rows, cols // 4).view(np.uint8).reshape(rows, cols)
     assert np.array_equal(out.cpu().numpy(), want)
-    assert not bool((sf == -1).all(dim=1).any())          # every row's words were written
+    # the word of group 4 * p + g (p: piece of 512 columns, g: its 128-column group) is written by lane 16 * g + (p mod P)
+    # of the wave that holds the piece, P pieces per wave, and is the XOR of the first word that lane loaded of each of
+    # the wave's pieces
+    P = 4 if cols % 2048 == 0 else 2
+    want_sf = np.zeros((rows, cols // 128), dtype=np.uint32)
+    for tile in range(cols // (P * 512)):
+        for j in range(P):
+            for g in range(4):
+                lane = 16 * g + j
+                fold = np.zeros(rows, dtype=np.uint32)
+                for r in range(P):
+                    fold ^= w[:, ((tile * P + r) * 512 + lane * 8) // 2]
+                want_sf[:, (tile * P + j) * 4 + g] = fold
+    assert np.array_equal(sf.cpu().numpy().view(np.uint32), want_sf)
 
 
 def test_stream_floor_rejects_bad_shapes():

@@ -38,11 +38,12 @@ def _run_both(lib, T, K, E, alignment, seed):
     assert rc == 0, lib.tk_strerror(rc)
     got = _buffers(T, K, E, R, -9)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # free device memory as the driver reports it (torch's own counters would only see torch's allocator)
+    before, before_torch = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
     rc = lib.tk_get_fused_mapping_static(idx.data_ptr(), T, K, E, alignment, R, *[b.data_ptr() for b in got], stream)
     assert rc == 0, lib.tk_strerror(rc)
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == before and torch.cuda.memory_allocated() == before_torch
     for name, g, w in zip(NAMES, got, want):
         assert torch.equal(g.cpu(), w.cpu()), (name, T, K, E, alignment)
     # the mapping is a bijection between the routed (token, k) pairs and the live positions
@@ -55,12 +56,16 @@ def _run_both(lib, T, K, E, alignment, seed):
 def test_static_scratch_mapping_matches_workspace_mapping_on_consecutive_calls():
     from tilekernels_amd import _ffi
     lib = _ffi.load()
-    # large first, then smaller inputs: the table keeps the earlier call's contents
+    # large first, then smaller inputs: the table keeps the earlier call's contents.  Lists of 64 Ki pairs or more, and
+    # more than 512 experts, take the three launches that go through the table; the others take the single launch
     _run_both(lib, 32768, 8, 256, 128, seed=1)     # 1024 slices x 256 experts = 1 MiB of the 4 MiB table
-    _run_both(lib, 20001, 8, 256, 64, seed=2)
-    _run_both(lib, 4001, 6, 72, 16, seed=3)
+    _run_both(lib, 20001, 8, 256, 64, seed=2)      # table
+    _run_both(lib, 9000, 8, 64, 16, seed=7)        # table: 72000 pairs, fewer experts than the calls before
+    _run_both(lib, 4001, 6, 72, 16, seed=3)        # single launch
     _run_both(lib, 7, 1, 1, 16, seed=4)
-    _run_both(lib, 16384, 8, 1024, 128, seed=5)    # 512 slices x 1024 experts = 2 MiB
+    _run_both(lib, 16384, 8, 1024, 128, seed=5)    # table: 512 slices x 1024 experts = 2 MiB
+    _run_both(lib, 1024, 8, 600, 16, seed=8)       # table (more than 512 experts) although the list is short
+    _run_both(lib, 8192, 8, 16, 32, seed=9)        # table: exactly 64 Ki pairs
     _run_both(lib, 513, 9, 32, 16, seed=6)
 
 

@@ -15,7 +15,7 @@ CSRC = os.path.join(PKG, 'csrc')
 LIB_DIR = os.path.join(PKG, 'lib')
 LIB_PATH = os.path.join(LIB_DIR, 'libtk_quant.so')
 SOURCES = ['api.hip', 'per_token_cast.hip', 'per_block_cast.hip', 'swiglu_cast.hip', 'cast_back.hip', 'moe_layout.hip',
-           'swiglu_backward.hip', 'per_channel_cast.hip', 'lossless_cast.hip', 'stream_floor.hip']
+           'swiglu_backward.hip', 'per_channel_cast.hip', 'lossless_cast.hip', 'stream_floor.hip', 'swiglu_cast_variants.hip']
 
 HIPCC = os.environ.get('HIPCC', '/opt/rocm/bin/hipcc')
 FLAGS = [

@@ -59,11 +59,19 @@ __device__ __forceinline__ void per_block_cast_tile(const PerBlockParams &p) {
     const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * p.K + col;
     const int64_t out_ld = FMT == TK_E4M3 ? p.K : p.K / 2;
 
+    // fp32 input: the LPR lanes of a tile row read its 32 * LPR bytes as two whole-line loads and deal them out through LDS
+    constexpr int XB = Raw8<InT>::kXchgBytes;
+    constexpr int RUN = LPR < 64 ? LPR : 64;     // lanes of one run: a tile row, or the part of it that one wave holds
+    __shared__ __attribute__((aligned(16))) uint8_t xchg[XB ? THREADS * XB : 16];
     Raw8<InT> raw[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-        if (FULL) raw[i].load(x + (int64_t)(TR * i) * p.K);
+        if (FULL) raw[i].template load_run<RUN>(x + (int64_t)(TR * i) * p.K, c % RUN);
         else raw[i].load(x + (int64_t)(TR * i) * p.K, col_ok && row0 + TR * i < p.M);
+    }
+    if constexpr (FULL && XB != 0) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) raw[i].template settle<RUN>(xchg + (threadIdx.x / RUN) * (RUN * XB), c % RUN);
     }
 
     float inv[SUBM];

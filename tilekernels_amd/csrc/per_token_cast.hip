@@ -76,6 +76,9 @@ __global__ __launch_bounds__(TILE == T_WIDE ? 64 * kMaxWideWaves : kThreads) voi
     const int nwaves = WIDE ? p.geom : kWaves;
     using RS = RowScales<Fmt<FMT>::qmax, RPW, LPG>;
     __shared__ uint32_t stage[ROWW ? 1 : ROWS][ROWW ? 1 : SGPR];
+    // fp32 input: a wave's 2 KB of one row arrive as two whole-line loads and are dealt out to their lanes through LDS
+    constexpr int XB = Raw8<InT>::kXchgBytes;
+    __shared__ __attribute__((aligned(16))) uint8_t xchg[XB ? (WIDE ? kMaxWideWaves : kWaves) : 1][XB ? 64 * XB : 16];
 
     // wide tiles: the waves of one tile cover a whole row; row-wise: one wave does
     const bool one_col = (ROWW ? RPW : p.geom) * kStripCols >= p.K;
@@ -101,7 +104,7 @@ __global__ __launch_bounds__(TILE == T_WIDE ? 64 * kMaxWideWaves : kThreads) voi
     for (int r = 0; r < RPW; ++r) {
         const void *xp = elem_ptr<InT>(p.x, row0 + r * kRowStep, p.x_ld, col + r * kColStep);
         if (FULL) {
-            raw[r].load(xp);
+            raw[r].template load_run<64>(xp, lane);
         } else {
             // no branch around the load (the loads of the wave's rows then go out together): a lane beyond the last
             // row or column reads the first bytes of the matrix and is cleared by value
@@ -114,6 +117,11 @@ __global__ __launch_bounds__(TILE == T_WIDE ? 64 * kMaxWideWaves : kThreads) voi
             const bool ok = col_ok && (FULL || row0 + r < p.M);
             raw[r].s = ok ? sf_load(p.xsf, (row0 + r * kRowStep) / p.in_bm, (col + r * kColStep) / p.in_bk) : 0.0f;
         }
+    }
+
+    if constexpr (FULL && XB != 0) {
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) raw[r].template settle<64>(xchg[wave], lane);
     }
 
     float inv[RPW];

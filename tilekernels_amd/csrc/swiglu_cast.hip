@@ -111,6 +111,9 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
     const int rows = DIRECT ? nwaves : ROWS;
     using RS = RowScales<448, RPW, 16>;
     __shared__ uint32_t stage[DIRECT ? 1 : ROWS][DIRECT ? 1 : SGPR];
+    // fp32 input: a wave's 2 KB of one row arrive as two whole-line loads and are dealt out to their lanes through LDS
+    constexpr int XB = Raw8<InT>::kXchgBytes;
+    __shared__ __attribute__((aligned(16))) uint8_t xchg[XB ? kWaves : 1][XB ? 64 * XB : 16];
 
     const int total = LOOP ? ((p.R + rows - 1) / rows) * p.tiles_k : 1;
     const int lane = threadIdx.x & 63, wave = wave_id();
@@ -157,8 +160,15 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
             const InT *xr = x + (int64_t)(r * kRowStep) * (2 * (int64_t)p.H) + r * kColStep;
             const bool piece_ok = FULL || col + r * kColStep < p.H;
             if (FULL && !MASK) {
-                rg[r].load(xr);
-                ru[r].load(xr + p.H);
+                rg[r].template load_run<64>(xr, lane);
+                ru[r].template load_run<64>(xr + p.H, lane);
+            } else if (FULL && XB != 0) {
+                // (a padding row reads the first 2 KB of the matrix, as one run)
+                const bool ok = live[r];
+                const InT *src = ok ? xr : reinterpret_cast<const InT *>(p.x) + lane * 8;
+                rg[r].template load_run<64>(src, lane);
+                ru[r].template load_run<64>(ok ? xr + p.H : src, lane);
+                if (!ok) { rg[r].zero(); ru[r].zero(); }
             } else {
                 // no branch around the loads (a branch would make the compiler wait for all eight loads
                 // before the first row is evaluated): a padding row, and a lane beyond the last row or column,
@@ -171,6 +181,13 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
             }
         }
 
+        if constexpr (FULL && XB != 0) {
+#pragma unroll
+            for (int r = 0; r < RPW; ++r) {
+                rg[r].template settle<64>(xchg[wave], lane);
+                ru[r].template settle<64>(xchg[wave], lane);
+            }
+        }
         float wrow = 0.0f;
         if constexpr (EARLY_WEIGHT) {
             if (has_weight && live[0] && wpos >= 0 && wpos < p.num_weights) wrow = uniform_load(p.topk_weights + wpos);
