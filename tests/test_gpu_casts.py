@@ -107,6 +107,26 @@ def test_per_block_cast(M, K, block, dtype, fmt, mode):
         assert_same(c3, torch_ref.cast(x, fmt, block, sf=sf_ref, **kw), 'codes from given sf')
 
 
+@pytest.mark.parametrize('mode', [(False, False, False), (True, True, True)], ids=_mode_id)
+@pytest.mark.parametrize('fmt', ['e4m3', 'e2m1'])
+@pytest.mark.parametrize('M,K,block', [(4096, 2048, (128, 128)), (3968, 2560, (32, 32)), (4230, 2048, (128, 32)), (2048, 4096, (32, 128))])
+def test_per_block_cast_wide_tiles(M, K, block, fmt, mode):
+    """bf16 matrices of 512 to 1280 tiles of 128 x 128 whose width is a multiple of 512 take tiles of 128 x 512, whose lane
+    pairs exchange codes and store 16 consecutive ones (8 bytes of FP4) each; a ragged last row of tiles takes the other path."""
+    tk = _tk()
+    col, rnd, packed = mode
+    x = _rand((M, K), torch.bfloat16)
+    xg = x.cuda()
+    kw = dict(use_tma_aligned_col_major_sf=col, round_sf=rnd, use_packed_ue8m0=packed)
+    codes, sf = tk.quant.per_block_cast(xg, fmt, block, **kw)
+    codes_ref, sf_ref = torch_ref.cast(x, fmt, block, **kw)
+    assert_same(sf, sf_ref, 'sf')
+    assert_same(codes, codes_ref, 'codes')
+    if not col:
+        c3 = tk.quant.per_block_cast_with_precomputed_sf(xg, fmt, block, sf=sf * 0.5, **kw)     # half the scale: values saturate
+        assert_same(c3, torch_ref.cast(x, fmt, block, sf=sf_ref * 0.5, **kw), 'codes from given sf')
+
+
 def _all_bf16_as_f32():
     v = (np.arange(65536, dtype=np.uint32) << 16).view(np.float32)
     return torch.from_numpy(v[np.isfinite(v)].copy())

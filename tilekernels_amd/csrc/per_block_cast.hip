@@ -14,6 +14,7 @@
 namespace tk {
 
 constexpr int kBlockTile = 128;
+constexpr int kPerBlockThreads = 512, kWideTile = 512, kWideThreads = 1024;   // the two tile shapes: see the table at the launch code
 
 struct PerBlockParams {
     const void *x;
@@ -115,6 +116,33 @@ __device__ __forceinline__ void per_block_cast_tile(const PerBlockParams &p) {
     }
     if (p.mode == TK_SF_ONLY) return;
 
+    // Wide tiles: the two lanes that hold 16 neighbouring columns exchange the codes of two row slots, so that each stores
+    // 16 consecutive codes of one row with one instruction: half as many store instructions, each twice as wide.  A launch of
+    // wide tiles fits the GPU in one round, all its workgroups finish loading at about the same time (measured: the last load
+    // of every workgroup of [7168, 2048] arrives between 3.4 and 4.7 us after the start) and the rest of the launch is one
+    // burst of stores, which drains faster in fewer, wider instructions: bf16 [7168, 2048] -> E4M3 8.54 -> 8.20 us,
+    // [4096, 4096] 9.22 -> 8.66, [8192, 2048] 9.94 -> 9.07.  (128-column tiles, whose workgroups finish at different times so
+    // that loads and stores overlap, do not gain: [8192, 4096] 17.43 -> 17.65 us.)
+    constexpr bool PAIRED = FULL && TW == kWideTile && NI % 2 == 0;
+    if constexpr (PAIRED) {
+        const bool odd = threadIdx.x & 1;
+#pragma unroll
+        for (int i = 0; i < NI; i += 2) {
+            float v[8];
+            raw[i].get(v);
+            const u32x2 a = p.mode == TK_CAST_GIVEN_SF ? quantise8<FMT, true>(v, inv[i / IPB]) : quantise8<FMT, false>(v, inv[i / IPB]);
+            raw[i + 1].get(v);
+            const u32x2 b = p.mode == TK_CAST_GIVEN_SF ? quantise8<FMT, true>(v, inv[(i + 1) / IPB]) : quantise8<FMT, false>(v, inv[(i + 1) / IPB]);
+            // the even lane keeps slot i and takes its neighbour's half of it, the odd lane likewise with slot i + 1
+            const u32x2 send = odd ? a : b;
+            const u32x2 recv = {dpp_u32<kDppXor1>(send.x), FMT == TK_E4M3 ? dpp_u32<kDppXor1>(send.y) : 0u};
+            const u32x2 lo = odd ? recv : a, hi = odd ? b : recv;
+            uint8_t *out_row = p.out + (int64_t)(row0 + TR * (i + (odd ? 1 : 0))) * out_ld;
+            if (FMT == TK_E4M3) st_stream16(out_row + (col & ~15), u32x4{lo.x, lo.y, hi.x, hi.y});
+            else st_stream8(out_row + ((col & ~15) >> 1), u32x2{lo.x, hi.x});
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
         const int row = row0 + TR * i;
@@ -154,7 +182,6 @@ __global__ __launch_bounds__(THREADS) void per_block_cast_kernel(TK_PB_KERNEL_AR
 // row per load instruction instead of 256 bytes of four rows, which pays while the matrix has too few 128 x 128
 // tiles to fill the GPU several times over (here 896 and 1024 tiles: 3.5 and 4 workgroups per CU) and costs where it
 // has many, or so few that whole CUs would stay empty.  The wide tile is used for bf16 input inside that window.
-constexpr int kPerBlockThreads = 512, kWideTile = 512, kWideThreads = 1024;
 constexpr int64_t kWideMinTiles = 512, kWideMaxTiles = 1280;     // in 128 x 128 tiles
 
 template <typename InT, int FMT, int BM, int BK, int TW, int THREADS>

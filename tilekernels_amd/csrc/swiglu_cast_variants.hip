@@ -26,10 +26,6 @@ namespace tk {
 
 enum { V_BASE = 0, V_PKFLOOR = 1, V_WIDEST = 2, V_PRIO = 3, V_PIECESF = 4, V_LATE = 5, V_AHEAD = 6, V_ROUNDS = 7 };
 
-__device__ __forceinline__ void st_stream16(void *p, u32x4 v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
-}
-
 // the eight activations of one lane's piece
 template <bool PKFLOOR> __device__ __forceinline__ void eval_piece(const u32x4 &gw, const u32x4 &uw, float (&v)[8]) {
     Raw8<bf16_t> rg, ru;

@@ -107,6 +107,10 @@ __device__ __forceinline__ void st_stream8(void *p, u32x2 v) {
     __hip_atomic_store(reinterpret_cast<uint64_t *>(p), __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_SYSTEM);
 }
+// (the 16-byte form has no builtin with these cache bits)
+__device__ __forceinline__ void st_stream16(void *p, u32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+}
 __device__ __forceinline__ void st_stream4(void *p, uint32_t v) {
     __hip_atomic_store(reinterpret_cast<uint32_t *>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
@@ -449,6 +453,16 @@ __device__ __forceinline__ u32x3 pack_e5m6x8(const float (&q)[8]) {
     return u32x3{(c01 << 20) | (c1 << 8) | (c2 >> 4),
                  (c2 << 28) | (c3 << 16) | (c4 << 4) | (c5 >> 8),
                  (c5 << 24) | (c6 << 12) | c7};
+}
+
+// scale 8 values and convert: the 8 E4M3 codes, or the 8 E2M1 codes in the first word (the second is 0)
+template <int FMT, bool CLAMP> __device__ __forceinline__ u32x2 quantise8(const float (&v)[8], float inv) {
+    static_assert(FMT == TK_E4M3 || FMT == TK_E2M1, "formats with whole-word codes");
+    float q[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) q[i] = v[i] * inv;
+    if (FMT == TK_E4M3) return pack_e4m3x8<CLAMP>(q);
+    return u32x2{pack_e2m1x8(q), 0u};
 }
 
 // scale 8 values, convert, store: 8 bytes (E4M3), 4 bytes (E2M1) or 12 bytes (E5M6) per lane
