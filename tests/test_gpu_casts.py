@@ -109,13 +109,14 @@ def test_per_block_cast(M, K, block, dtype, fmt, mode):
 
 @pytest.mark.parametrize('mode', [(False, False, False), (True, True, True)], ids=_mode_id)
 @pytest.mark.parametrize('fmt', ['e4m3', 'e2m1'])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
 @pytest.mark.parametrize('M,K,block', [(4096, 2048, (128, 128)), (3968, 2560, (32, 32)), (4230, 2048, (128, 32)), (2048, 4096, (32, 128))])
-def test_per_block_cast_wide_tiles(M, K, block, fmt, mode):
-    """bf16 matrices of 512 to 1280 tiles of 128 x 128 whose width is a multiple of 512 take tiles of 128 x 512, whose lane
+def test_per_block_cast_wide_tiles(M, K, block, dtype, fmt, mode):
+    """Matrices of 512 to 1280 tiles of 128 x 128 whose width is a multiple of 512 take tiles of 128 x 512, whose lane
     pairs exchange codes and store 16 consecutive ones (8 bytes of FP4) each; a ragged last row of tiles takes the other path."""
     tk = _tk()
     col, rnd, packed = mode
-    x = _rand((M, K), torch.bfloat16)
+    x = _rand((M, K), dtype)
     xg = x.cuda()
     kw = dict(use_tma_aligned_col_major_sf=col, round_sf=rnd, use_packed_ue8m0=packed)
     codes, sf = tk.quant.per_block_cast(xg, fmt, block, **kw)

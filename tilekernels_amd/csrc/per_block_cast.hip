@@ -181,7 +181,8 @@ __global__ __launch_bounds__(THREADS) void per_block_cast_kernel(TK_PB_KERNEL_AR
 // (128 x 128 with 256 threads: 9.4 at [7168,2048], with 1024: 9.8.)  A wave of a 512-column tile reads 1 KB of one
 // row per load instruction instead of 256 bytes of four rows, which pays while the matrix has too few 128 x 128
 // tiles to fill the GPU several times over (here 896 and 1024 tiles: 3.5 and 4 workgroups per CU) and costs where it
-// has many, or so few that whole CUs would stay empty.  The wide tile is used for bf16 input inside that window.
+// has many, or so few that whole CUs would stay empty.  The wide tile is used inside that window (with the paired
+// 16-byte stores: [7168,2048] 8.24).  fp32 input, same window: [7168,2048] 13.58 -> 12.31, [8192,4096] 30.16 -> 29.96.
 constexpr int64_t kWideMinTiles = 512, kWideMaxTiles = 1280;     // in 128 x 128 tiles
 
 template <typename InT, int FMT, int BM, int BK, int TW, int THREADS>
@@ -196,7 +197,7 @@ static void launch_per_block_3(const PerBlockParams &p, hipStream_t stream) {
 template <typename InT, int FMT, int BM, int BK>
 static void launch_per_block_2(const PerBlockParams &p, hipStream_t stream) {
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_k;
-    if (sizeof(InT) == 2 && p.K % kWideTile == 0 && tiles >= kWideMinTiles && tiles <= kWideMaxTiles)
+    if (p.K % kWideTile == 0 && tiles >= kWideMinTiles && tiles <= kWideMaxTiles)
         launch_per_block_3<InT, FMT, BM, BK, kWideTile, kWideThreads>(p, stream);
     else
         launch_per_block_3<InT, FMT, BM, BK, kBlockTile, kPerBlockThreads>(p, stream);
