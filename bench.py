@@ -337,7 +337,7 @@ def launch_timeline(cfg: int, launches: int = 14, preheat_ms: float = 40.0) -> d
     }
 
 
-VARIANTS = {'base': 0, 'pkfloor': 1, 'widest': 2, 'prio': 3, 'piecesf': 4, 'late': 5, 'ahead': 6, 'rounds': 7}
+VARIANTS = {'base': 0, 'pkfloor': 1, 'widest': 2, 'prio': 3, 'piecesf': 4, 'late': 5, 'ahead': 6, 'rounds': 7, 'tail': 8}
 
 
 def variant_ab(specs, steps: int, rounds: int = 4, preheat_ms: float = 40.0) -> dict:

@@ -34,8 +34,10 @@ class Op:
     """`build()` returns (callable launching one call on torch's current stream, algorithmic bytes,
     footprint bytes of the buffer set, factory of a callable that runs the CPU oracle on the same input)."""
 
-    def __init__(self, name, workload, build):
-        self.name, self.workload, self.build = name, workload, build
+    def __init__(self, name, workload, build, floor=None):
+        # floor: (bytes read, bytes a lane reads per piece, bytes it writes per piece, pieces per wave) of the traffic-only
+        # kernel (tk_stream_floor_flat) that moves this operator's code and value bytes in loads and stores of its widths
+        self.name, self.workload, self.build, self.floor = name, workload, build, floor
 
 
 def _sets_needed(footprint: int) -> int:
@@ -476,45 +478,74 @@ def op_reduce_fused(fp8):
 OPS = [
     Op('reduce_fused', 'reduce_fused bf16 [R,4096] -> bf16 [4096,4096], top-8 of 256 experts, weighted', op_reduce_fused(False)),
     Op('reduce_fused_fp8', 'reduce_fused bf16 [R,4096] -> e4m3 [4096,4096] with output scale, top-8, weighted', op_reduce_fused(True)),
-    Op('per_block_cast_lossless', 'per_block_cast_lossless e2m1 1x32 (packed scales) -> e4m3 128x128, [7168,2048]', op_lossless),
+    Op('per_block_cast_lossless', 'per_block_cast_lossless e2m1 1x32 (packed scales) -> e4m3 128x128, [7168,2048]', op_lossless, floor=(7168 * 2048 // 2, 8, 16, 4)),
     Op('per_token_cast_e5m6', "per_token_cast fmt='e5m6' (12-bit, one scale per row) round_sf, bf16 [8192,4096]", op_e5m6('cast')),
     Op('cast_back_e5m6', 'cast_back of e5m6 -> bf16, [8192,4096]', op_e5m6('back')),
     Op('per_token_cast_k576', 'per_token_cast e4m3 1x64, short rows: bf16 [65536,576]', op_short_rows('cast')),
     Op('cast_back_k576', 'cast_back e4m3 1x64 -> bf16, short rows: [65536,576]', op_short_rows('back')),
-    Op('per_token_cast_with_sf_only', 'per_token_cast_with_sf_only e4m3 1x128, bf16 [4096,7168]', op_cast_variant('token', 'sf_only')),
+    Op('per_token_cast_with_sf_only', 'per_token_cast_with_sf_only e4m3 1x128, bf16 [4096,7168]', op_cast_variant('token', 'sf_only'), floor=(4096 * 7168 * 2, 16, 0, 2)),
     Op('per_token_cast_with_precomputed_sf', 'per_token_cast_with_precomputed_sf e4m3 1x128, bf16 [4096,7168]',
        op_cast_variant('token', 'given_sf')),
-    Op('per_block_cast_with_sf_only', 'per_block_cast_with_sf_only e4m3 128x128, bf16 [7168,2048]', op_cast_variant('block', 'sf_only')),
+    Op('per_block_cast_with_sf_only', 'per_block_cast_with_sf_only e4m3 128x128, bf16 [7168,2048]', op_cast_variant('block', 'sf_only'), floor=(7168 * 2048 * 2, 16, 0, 8)),
     Op('per_block_cast_with_precomputed_sf', 'per_block_cast_with_precomputed_sf e4m3 128x128, bf16 [7168,2048]',
-       op_cast_variant('block', 'given_sf')),
+       op_cast_variant('block', 'given_sf'), floor=(7168 * 2048 * 2, 16, 8, 8)),
     Op('swiglu_forward_and_per_token_cast_weighted',
        'swiglu_forward_and_per_token_cast e4m3 1x128, MoE-expanded bf16 [R,4096] with mask and routing weights', op_swiglu_weighted),
     Op('swiglu_forward_and_per_token_cast_packed_sf', 'swiglu_forward_and_per_token_cast e4m3 1x128, packed UE8M0 column-major scales, bf16 [8192,4096]',
        op_swiglu_dense(8192, 2048, True)),
     Op('swiglu_forward_and_per_token_cast_h768', 'swiglu_forward_and_per_token_cast e4m3 1x128, short rows: bf16 [32768,1536]',
-       op_swiglu_dense(32768, 768, False)),
+       op_swiglu_dense(32768, 768, False), floor=(32768 * 1536 * 2, 16, 4, 4)),
     Op('expand_to_fused_with_sf', 'expand_to_fused_with_sf e4m3 [4096,4096] + 1x128 scales -> [R,4096], top-8 of 256 experts, pad 128',
        op_expand_to_fused_with_sf),
     Op('cast_back', 'cast_back e4m3 1x128 -> bf16, [8192,4096]', op_cast_back('bf16')),
     Op('cast_back_fp32', 'cast_back e4m3 1x128 -> fp32, [8192,4096]', op_cast_back('fp32')),
-    Op('per_token_cast_quantized', 'per_token_cast of (e4m3 1x128) input -> e2m1 1x32, [8192,4096]', op_requant),
+    Op('per_token_cast_quantized', 'per_token_cast of (e4m3 1x128) input -> e2m1 1x32, [8192,4096]', op_requant, floor=(8192 * 4096, 16, 8, 2)),
     Op('get_fused_mapping', 'get_fused_mapping 4096 tokens, top-8 of 256 experts, pad 128', op_get_fused_mapping),
     Op('expand_to_fused', 'expand_to_fused bf16 [4096,4096] -> [R,4096], top-8 of 256 experts, pad 128', op_expand_to_fused),
     Op('swiglu_backward_and_per_token_cast', 'swiglu_backward_and_per_token_cast 1x128 round_sf, x e4m3 [8192,4096]',
        op_swiglu_backward(128)),
     Op('swiglu_backward_and_per_token_cast_g32', 'swiglu_backward_and_per_token_cast 1x32 round_sf, x e4m3 [8192,4096]',
        op_swiglu_backward(32)),
-    Op('per_channel_cast', 'per_channel_cast 128x1 round_sf, bf16 [8192,4096]', op_per_channel('bf16', False)),
+    Op('per_channel_cast', 'per_channel_cast 128x1 round_sf, bf16 [8192,4096]', op_per_channel('bf16', False), floor=(8192 * 4096 * 2, 16, 8, 8)),
     Op('per_channel_cast_fused_fp8_input', 'per_channel_cast_fused 128x1 of (e4m3 1x128) input, [8192,4096]',
-       op_per_channel('e4m3', False)),
+       op_per_channel('e4m3', False), floor=(8192 * 4096, 16, 16, 8)),
     Op('per_channel_cast_and_transpose', 'per_channel_cast_and_transpose 128x1 round_sf, bf16 [8192,4096] -> [4096,8192]',
-       op_per_channel('bf16', True)),
+       op_per_channel('bf16', True), floor=(8192 * 4096 * 2, 16, 8, 8)),
     Op('swiglu_forward_and_per_channel_cast_and_transpose',
        'swiglu_forward_and_per_channel_cast_and_transpose 128x1 round_sf, bf16 [8192,4096] -> [2048,8192]',
-       op_per_channel('swiglu', True, hidden=2048)),
+       op_per_channel('swiglu', True, hidden=2048), floor=(8192 * 4096 * 2, 16, 4, 8)),
     Op('swiglu_forward_and_per_channel_cast', 'same without transpose, bf16 [8192,4096] -> [8192,2048]',
-       op_per_channel('swiglu', False, hidden=2048)),
+       op_per_channel('swiglu', False, hidden=2048), floor=(8192 * 4096 * 2, 16, 4, 8)),
 ]
+
+
+def time_floor(spec, steps: int, warmup: int) -> dict:
+    """The traffic-only kernel on flat buffers of the operator's size, rotated past the last-level cache like the
+    operator's own: what the same bytes cost on this machine in loads and stores of the same widths, with no arithmetic."""
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    in_bytes, ipl, opl, pieces = spec
+    out_bytes = in_bytes // ipl * opl
+    n = _sets_needed(in_bytes + out_bytes)
+    ins = [torch.randint(0, 255, (in_bytes,), dtype=torch.uint8, device='cuda') for _ in range(n)]
+    outs = [torch.empty((max(out_bytes, 16),), dtype=torch.uint8, device='cuda') for _ in range(n)]
+    stream = _ffi.current_stream(ins[0].device)
+
+    def launch(i):
+        rc = lib.tk_stream_floor_flat(ins[i % n].data_ptr(), in_bytes, ipl, outs[i % n].data_ptr() if opl else 0, opl, pieces, stream)
+        assert rc == 0, rc
+    for i in range(warmup):
+        launch(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        launch(i)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / steps
+    return {'us_per_call': round(us, 2), 'bytes': in_bytes + out_bytes, 'frac': round((in_bytes + out_bytes) / us / 1e3 / HBM_PEAK_GBS, 4),
+            'what': f'tk_stream_floor_flat: {in_bytes} bytes read in {ipl}-byte loads, {out_bytes} written in {opl}-byte stores, {pieces} pieces per wave'}
 
 
 def time_cpu(make) -> dict:
@@ -553,6 +584,11 @@ def run(op: Op, steps: int, warmup: int, with_cpu: bool) -> dict:
     gbs = algo / us / 1e3
     rec = {'op': op.name, 'workload': op.workload, 'us_per_call': round(us, 2), 'bytes': algo, 'GB/s': round(gbs, 1),
            'frac': round(gbs / HBM_PEAK_GBS, 4), 'buffer_sets': n, 'steps': steps, 'warmup': warmup}
+    if op.floor is not None:
+        del sets
+        torch.cuda.empty_cache()
+        rec['traffic_only_kernel'] = time_floor(op.floor, steps, warmup)
+        rec['over_traffic_only'] = round(us / rec['traffic_only_kernel']['us_per_call'], 3)
     if with_cpu:
         rec['cpu_baseline'] = time_cpu(make_cpu)
     return rec

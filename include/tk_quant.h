@@ -344,6 +344,17 @@ int tk_stream_floor_timeline(const void *x, int64_t rows, int64_t cols, int two_
 int64_t tk_stream_floor_stamp_words(int64_t rows, int64_t cols);
 
 /*
+ * tk_stream_floor_flat: the traffic-only kernel for any ratio of bytes read to bytes written (measurement aid, no
+ * counterpart in the reference; bench_ops.py times it beside the operators around the path).  The input is a flat range of
+ * in_bytes bytes; a lane reads in_bytes_per_lane (16, 8 or 4) bytes per piece of 64 lanes and writes out_bytes_per_lane
+ * (16, 8, 4 or 0) bytes per piece to the flat output; a wave takes pieces_per_wave (1, 2, 4 or 8) consecutive pieces, all
+ * its loads issued before its first store.  What is written is an XOR fold of what was read.
+ *   requirements in_bytes % (64 * in_bytes_per_lane) == 0; in and out 16-byte aligned
+ */
+int tk_stream_floor_flat(const void *in, int64_t in_bytes, int in_bytes_per_lane, void *out, int out_bytes_per_lane,
+                         int pieces_per_wave, void *stream);
+
+/*
  * tk_swiglu_cast_variant: measurement aid with no counterpart in the reference.  Alternative structures of the kernel
  * behind tk_swiglu_per_token_cast for its plain case (bf16 x[R, 2H], E4M3 codes, row-major fp32 1 x 128 scales, no mask,
  * weights or clamp), each producing the same codes and scales bit for bit; bench.py --variant times them beside the
@@ -353,6 +364,7 @@ int64_t tk_stream_floor_stamp_words(int64_t rows, int64_t cols);
  *   2 16-byte code stores after a lane-pair exchange (param as 0)                  5 variant 4 for waves whose first piece
  *   3 wave priority raised once the first piece has arrived (param as 0)             arrives later than param * 10 ns
  *   6 pieces requested param (1, 2) ahead instead of all at once                   7 param (1, 2) pieces per wave, not 4
+ *   8 the last param per cent of the rows as four one-piece waves each (H = 2048)
  *   requirements H % 2048 == 0, R % 8 == 0; x and out 16-byte aligned
  */
 int tk_swiglu_cast_variant(const void *x, int64_t R, int64_t H, void *out, void *sf, int variant, int param, void *stream);

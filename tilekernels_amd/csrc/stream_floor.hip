@@ -68,9 +68,82 @@ __global__ __launch_bounds__(kThreads) void stream_floor_kernel(const bf16_t *x,
     }
 }
 
+// The same idea for any ratio of bytes read to bytes written: a lane reads IN (16, 8 or 4) bytes per piece and writes OUT
+// (16, 8, 4 or 0) bytes per piece, a piece being 64 lanes side by side; a wave takes PIECES consecutive pieces, all loads
+// issued before the first store.  Input and output are flat byte ranges.
+template <int IN> __device__ __forceinline__ u32x4 floor_load(const uint8_t *p) {
+    if constexpr (IN == 16) return ld_stream16(p);
+    else if constexpr (IN == 8) { const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p)); return u32x4{v.x, v.y, 0u, 0u}; }
+    else { const uint32_t v = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p)); return u32x4{v, 0u, 0u, 0u}; }
+}
+template <int OUT> __device__ __forceinline__ void floor_store(uint8_t *p, u32x4 v) {
+    if constexpr (OUT == 16) st_stream16(p, v);
+    else if constexpr (OUT == 8) st_stream8(p, u32x2{v.x ^ v.z, v.y ^ v.w});
+    else if constexpr (OUT == 4) st_stream4(p, v.x ^ v.y ^ v.z ^ v.w);
+}
+
+template <int IN, int OUT, int PIECES>
+__global__ __launch_bounds__(kThreads) void stream_floor_flat_kernel(const uint8_t *in, int64_t pieces, uint8_t *out, uint32_t *sink) {
+    const int lane = threadIdx.x & 63;
+    const int64_t first = ((int64_t)blockIdx.x * kWaves + wave_id()) * PIECES;
+    if (first >= pieces) return;
+    u32x4 v[PIECES];
+#pragma unroll
+    for (int r = 0; r < PIECES; ++r) {
+        const int64_t piece = first + r < pieces ? first + r : first;       // (a wave's surplus pieces read its first again)
+        v[r] = floor_load<IN>(in + (piece * 64 + lane) * IN);
+    }
+    uint32_t fold = 0;
+#pragma unroll
+    for (int r = 0; r < PIECES; ++r) {
+        if (OUT != 0 && first + r < pieces) floor_store<OUT>(out + ((first + r) * 64 + lane) * OUT, v[r]);
+        fold ^= v[r].x ^ v[r].y ^ v[r].z ^ v[r].w;
+    }
+    // nothing written: the loads must still be used.  No fold of real data is ever this value in all lanes at once
+    if (OUT == 0 && fold == 0x9E3779B9u && sink != nullptr) st_stream4(sink, fold);
+}
+
 }  // namespace tk
 
 using namespace tk;
+
+extern "C" int tk_stream_floor_flat(const void *in, int64_t in_bytes, int in_bytes_per_lane, void *out, int out_bytes_per_lane,
+                                    int pieces_per_wave, void *stream) {
+    const int I = in_bytes_per_lane, O = out_bytes_per_lane, P = pieces_per_wave;
+    if ((I != 16 && I != 8 && I != 4) || (O != 16 && O != 8 && O != 4 && O != 0) || (P != 1 && P != 2 && P != 4 && P != 8)) return TK_ERR_BAD_MODE;
+    if (in_bytes < 0 || in_bytes % (64 * I) != 0) return TK_ERR_BAD_SHAPE;
+    if (in_bytes == 0) return TK_OK;
+    if (!in || (O != 0 && !out)) return TK_ERR_NULL_POINTER;
+    if (!aligned_to(in, 16) || !aligned_to(out, 16)) return TK_ERR_MISALIGNED;
+    const int64_t pieces = in_bytes / (64 * I), waves = (pieces + P - 1) / P, blocks = (waves + kWaves - 1) / kWaves;
+    if (blocks > INT32_MAX) return TK_ERR_TOO_LARGE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint8_t *ip = static_cast<const uint8_t *>(in);
+    uint8_t *op = static_cast<uint8_t *>(out);
+#define TK_FLAT_3(II, OO, PP) \
+    hipLaunchKernelGGL((stream_floor_flat_kernel<II, OO, PP>), dim3((unsigned)blocks), dim3(kThreads), 0, s, ip, pieces, op, (uint32_t *)nullptr)
+#define TK_FLAT_2(II, OO)                 \
+    do {                                  \
+        if (P == 1) TK_FLAT_3(II, OO, 1); \
+        else if (P == 2) TK_FLAT_3(II, OO, 2); \
+        else if (P == 4) TK_FLAT_3(II, OO, 4); \
+        else TK_FLAT_3(II, OO, 8);        \
+    } while (0)
+#define TK_FLAT_1(II)                     \
+    do {                                  \
+        if (O == 16) TK_FLAT_2(II, 16);   \
+        else if (O == 8) TK_FLAT_2(II, 8); \
+        else if (O == 4) TK_FLAT_2(II, 4); \
+        else TK_FLAT_2(II, 0);            \
+    } while (0)
+    if (I == 16) TK_FLAT_1(16);
+    else if (I == 8) TK_FLAT_1(8);
+    else TK_FLAT_1(4);
+#undef TK_FLAT_1
+#undef TK_FLAT_2
+#undef TK_FLAT_3
+    return (int)hipGetLastError();
+}
 
 static int stream_floor_launch(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, void *stamps,
                                bool stamp, void *stream) {

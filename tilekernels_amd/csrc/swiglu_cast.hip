@@ -9,6 +9,8 @@
 //
 // Reference semantics: tile_kernels/quant/swiglu_forward_and_per_token_cast_kernel.py:61-170,
 // tile_kernels/torch/swiglu.py:62-86.
+#include <algorithm>
+
 #include "swiglu_math.hpp"
 #include "tk_device.hpp"
 #include "tk_host.hpp"
@@ -33,18 +35,24 @@ struct SwigluParams {
 
 // The kernels take their parameters as individual scalars in the order they are needed: the leading
 // 14 dwords of the kernel-argument segment arrive preloaded in SGPRs when a wave starts (the library is
-// built with -amdgpu-kernarg-preload-count=16) and hold everything the input addresses are made of; the
-// others are fetched from the argument buffer (host memory) while the first loads are in flight.
+// built with -amdgpu-kernarg-preload-count=16) and hold everything the input addresses are made of, plus the two
+// values that every code path of the tiled kernel uses (the compiler computes what all paths share before the
+// first branch, and would wait there for an argument that is not preloaded); the others are fetched from the
+// argument buffer (host memory) while the first loads are in flight.
 #define TK_SWIGLU_KERNEL_ARGS                                                                                      \
     const void *a_x, const int32_t *a_pe, int a_R, int a_H, int a_nwaves, int a_tiles_k, uint8_t *a_out, void *a_sf, \
-        int64_t a_sf_ld, float a_floor, float a_clamp, int a_round_sf, int a_sf_layout, const int32_t *a_ptt,          \
+        float a_floor, int a_round_sf, int64_t a_sf_ld, float a_clamp, int a_sf_layout, const int32_t *a_ptt,          \
         const float *a_w, unsigned long long *a_cnt, int64_t a_nw, int a_nk
 #define TK_SWIGLU_KERNEL_UNPACK                                                                            \
     const SwigluParams p{a_x, a_out, SfRef{a_sf, a_sf_ld, a_sf_layout, a_R, a_nk}, a_ptt, a_w, a_pe, a_cnt, \
                          a_nw, a_R, a_H, a_nwaves, a_tiles_k, a_round_sf, a_floor, a_clamp}
+// (the variant whose later arguments are fetched behind the loads: see fetch_late_arguments)
+#define TK_SWIGLU_KERNEL_UNPACK_EARLY                                                                                   \
+    SwigluParams p{a_x, a_out, SfRef{a_sf, (int64_t)reinterpret_cast<intptr_t>(a_pe), TK_SF_ROW_F32, a_R, 0}, nullptr, nullptr, \
+                   nullptr, nullptr, 0, a_R, a_H, a_nwaves, a_tiles_k, a_round_sf, a_floor, 0.0f}
 #define TK_SWIGLU_LAUNCH_ARGS(p)                                                                                  \
-    (p).x, (p).pos_to_expert, (p).R, (p).H, (p).nwaves, (p).tiles_k, (p).out, (p).sf.base, (p).sf.ld, (p).floor_,  \
-        (p).clamp, (p).round_sf, (p).sf.layout, (p).pos_to_token_topk, (p).topk_weights, (p).clamped_count,         \
+    (p).x, (p).pos_to_expert, (p).R, (p).H, (p).nwaves, (p).tiles_k, (p).out, (p).sf.base, (p).floor_, (p).round_sf, \
+        (p).sf.ld, (p).clamp, (p).sf.layout, (p).pos_to_token_topk, (p).topk_weights, (p).clamped_count,            \
         (p).num_weights, (p).sf.nk
 
 // CLAMP: 0 none, 1 clamp, 2 clamp and count
@@ -70,10 +78,89 @@ template <int CLAMP> struct ClampCounter {
     }
 };
 
+// The kernel-argument segment of TK_SWIGLU_KERNEL_ARGS, field for field.
+struct SwigluLateKernargs {
+    int64_t sf_ld; float clamp; int sf_layout; const int32_t *ptt; const float *w; unsigned long long *cnt; int64_t nw; int nk;
+};
+struct SwigluKernargs {
+    const void *x; const int32_t *pe; int R, H, nwaves, tiles_k; uint8_t *out; void *sf; float floor_; int round_sf;
+    SwigluLateKernargs late;
+};
+
+// The arguments beyond the preloaded ones that the row-wise waves use after their vector loads, read from the argument
+// segment here and now.  A kernel whose code paths part before the loads names these arguments nowhere else: named, their
+// fetch and the first arithmetic on them (a null test, an address) would be placed where the paths still run together,
+// i.e. in front of the loads, and every wave would wait for the fetch before it requests its data.  Each wave pays a round
+// trip to the scalar cache per argument it looks at here, one after the other where a later one is only fetched if an
+// earlier one says so; for the one- and two-piece waves at the end of a launch that is time their data does not cover
+// (bf16 [8192, 2 x 2048]: 14.7 us with the routing arguments looked at by every wave, 14.3 us without), so only what the
+// variant at hand uses is fetched: the clamp value, the routing list with its weights and their count.  (The leading
+// dimension of the scales, which every wave needs, travels in a preloaded place: see the launch code.)
+__device__ __forceinline__ void fetch_late_arguments(SwigluParams &p, bool with_clamp, bool with_weights) {
+    uintptr_t ka = (uintptr_t)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(ka) : : "memory");      // stays behind the loads issued before it
+    const SwigluLateKernargs *k = &reinterpret_cast<const SwigluKernargs *>(ka)->late;
+    if (with_clamp) p.clamp = uniform_load(&k->clamp);
+    if (with_weights) {
+        p.pos_to_token_topk = uniform_load(&k->ptt);
+        p.topk_weights = uniform_load(&k->w);
+        p.num_weights = uniform_load(&k->nw);
+    }
+}
+
 // `row` must be wave-uniform
 __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
     const int pos = uniform_load(p.pos_to_token_topk + row);
     return (pos >= 0 && pos < p.num_weights) ? uniform_load(p.topk_weights + pos) : 0.0f;
+}
+
+// One wave on NP consecutive pieces of one row (row-major scales, which the wave stores itself; no mask; CLAMP 0 or 1):
+// what a wave of a T_ROW tile does, for the finer-grained waves at the end of a launch (see the tiled kernel).
+template <typename InT, int CLAMP, int NP, bool WEIGHTED>
+__device__ __forceinline__ void swiglu_row_wave(SwigluParams p, int row0, int strip) {
+    static_assert(CLAMP != 2, "the counting variant loops over tiles");
+    static_assert(Raw8<InT>::kXchgBytes == 0, "inputs whose pieces need no exchange between lanes");
+    constexpr int GPS = kStripCols / 128;
+    using RS = RowScales<448, NP, 16>;
+    const int lane = threadIdx.x & 63, own = lane & 15;
+    const int col = strip * kStripCols + lane * 8;
+    const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * (2 * (int64_t)p.H) + col;
+    Raw8<InT> rg[NP], ru[NP];
+#pragma unroll
+    for (int r = 0; r < NP; ++r) {
+        rg[r].load(x + r * kStripCols);
+        ru[r].load(x + r * kStripCols + p.H);
+    }
+    fetch_late_arguments(p, CLAMP != 0, WEIGHTED);
+    const float w = WEIGHTED ? row_weight(p, row0) : 0.0f;
+    ClampCounter<CLAMP> clamp;
+    float v[NP][8], amax[NP];
+#pragma unroll
+    for (int r = 0; r < NP; ++r) {
+        float g[8], u[8];
+        rg[r].get(g);
+        ru[r].get(u);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            clamp.apply(g[i], u[i], p.clamp);
+            v[r][i] = silu_mul<InT>(g[i], u[i]);
+        }
+        if (WEIGHTED) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[r][i] = v[r][i] * w;
+        }
+        amax[r] = group_allmax<16>(absmax8(v[r]));
+    }
+    RS rs;
+    rs.compute(amax, p.floor_, p.round_sf != 0, lane);
+    // lane j (< A) of a group computed the scale of piece c*A + j; the wave's scales form one run of NP * 4 floats
+    if (own < RS::A) {
+#pragma unroll
+        for (int c = 0; c < RS::NC; ++c)
+            st_stream4(reinterpret_cast<float *>(p.sf.base) + (int64_t)row0 * p.sf.ld + (strip + c * RS::A + own) * GPS + (lane >> 4), f2u(rs.own[c].sf));
+    }
+#pragma unroll
+    for (int r = 0; r < NP; ++r) quantise_store8<TK_E4M3, false>(v[r], rs.inv[r], p.out + (int64_t)row0 * p.H, col + r * kStripCols);
 }
 
 // Tile shapes (a wave always holds RPW pieces of 512 output columns, each with its gate and its up half):
@@ -91,9 +178,52 @@ __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
 enum { T_STACKED = 0, T_ROW = 2, T_ROWC = 3 };
 
 // ONECOL: the grid is known to be a single column of tiles (else it is found out at run time)
-template <typename InT, int CLAMP, int RPW, int TILE, bool FULL_GRID, bool MASK, bool ONECOL>
+// TAILED (T_ROW tiles of four-piece waves, exact grids): the launch ends in finer-grained waves.  The grid's row tiles
+// come in three runs: `yb` workgroups of one-row waves as described above, then `ym` workgroups whose waves take two
+// pieces, then workgroups whose waves take one; all cover the rows in order.  The requests of a launch are served
+// roughly in the order they were made, so what arrives last belongs to the last workgroups; with whole rows per wave
+// the launch ends with the few waves that got their data last each working through a whole row alone on its SIMD while
+// the rest of the GPU is idle, with small waves that work is spread over four times as many SIMDs, and the small waves
+// start in the slots that finished waves free, so the second half of the bytes is requested while the first is being
+// served.  Measured on MI355X, bf16 [8192, 2 x 2048] (us per call): all rows by one-row waves 14.55; the last 40 % of
+// the rows by two-piece waves 14.35; by one-piece waves 14.35 - 14.45; the last 70 % in two-piece and of those the last
+// 15 % in one-piece waves 14.06 (55 % / 15 % of the rows: 2.2 and 0.6 times the GPU's wave slots).  The arguments pack
+// the run lengths into the two tile-geometry words (see the launch code) so that they arrive preloaded, and the place of
+// the mask pointer (these launches have no mask) carries the leading dimension of the scales.  TAILED: 1 without, 2 with
+// routing weights.
+template <typename InT, int CLAMP, int RPW, int TILE, bool FULL_GRID, bool MASK, bool ONECOL, int TAILED = 0>
 __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
-    TK_SWIGLU_KERNEL_UNPACK;
+    static_assert(!TAILED || (TILE == T_ROW && FULL_GRID && !MASK && CLAMP != 2 && RPW == 4), "tail waves: exact unmasked grids of one-row waves of four pieces");
+    if constexpr (TAILED) {
+        // a_nwaves: waves per workgroup (bits 0-3), column tiles (4-15), two-piece workgroups (16-31); a_tiles_k: one-row workgroups
+        const int yb = a_tiles_k, ym = (int)((unsigned)a_nwaves >> 16);
+        a_tiles_k = (a_nwaves >> 4) & 0xFFF;
+        a_nwaves &= 15;
+        const bool one_col = ONECOL || a_tiles_k == 1;
+        const int y = tile_grid_row(one_col);
+        if (y >= yb) {
+            TK_SWIGLU_KERNEL_UNPACK_EARLY;
+            const int strip0 = tile_grid_col(one_col) * RPW, wave = wave_id();
+            const int rb = yb * p.nwaves;                       // rows done by one-row waves
+            int row, strip;
+            if (y - yb < ym) {
+                const int sub = (y - yb) * p.nwaves + wave;     // two waves per row
+                row = rb + (sub >> 1);
+                strip = strip0 + (sub & 1) * 2;
+                swiglu_row_wave<InT, CLAMP, 2, TAILED == 2>(p, row, strip);
+            } else {
+                const int sub = (y - yb - ym) * p.nwaves + wave;      // four waves per row
+                row = rb + ((ym * p.nwaves) >> 1) + (sub >> 2);
+                strip = strip0 + (sub & 3);
+                if (row < p.R) swiglu_row_wave<InT, CLAMP, 1, TAILED == 2>(p, row, strip);    // (the grid may overhang along z)
+            }
+            return;
+        }
+    }
+    SwigluParams p = TAILED ? SwigluParams{a_x, a_out, SfRef{a_sf, (int64_t)reinterpret_cast<intptr_t>(a_pe), TK_SF_ROW_F32, a_R, 0}, nullptr, nullptr,
+                                           nullptr, nullptr, 0, a_R, a_H, a_nwaves, a_tiles_k, a_round_sf, a_floor, 0.0f}
+                            : SwigluParams{a_x, a_out, SfRef{a_sf, a_sf_ld, a_sf_layout, a_R, a_nk}, a_ptt, a_w, a_pe, a_cnt,
+                                           a_nw, a_R, a_H, a_nwaves, a_tiles_k, a_round_sf, a_floor, a_clamp};
     // T_ROW tiles always fit the columns, and their waves share nothing: on a grid that overhangs the last row the waves
     // beyond it leave at once and the others run without bounds checks, like on an exact grid
     constexpr bool ROWGUARD = TILE == T_ROW && !FULL_GRID && CLAMP != 2;
@@ -117,7 +247,7 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
 
     const int total = LOOP ? ((p.R + rows - 1) / rows) * p.tiles_k : 1;
     const int lane = threadIdx.x & 63, wave = wave_id();
-    const bool has_weight = p.pos_to_token_topk != nullptr;
+    const bool has_weight = TAILED ? TAILED == 2 : p.pos_to_token_topk != nullptr;
     const int own = lane & 15;
     const int srow = ROWC ? wave : wave * RPW;
     ClampCounter<CLAMP> counter;
@@ -181,6 +311,8 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
             }
         }
 
+        // (in this variant the fetch of the later arguments starts at the head of the kernel, where its paths part)
+        if constexpr (TAILED != 0) fetch_late_arguments(p, CLAMP != 0, TAILED == 2);
         if constexpr (FULL && XB != 0) {
 #pragma unroll
             for (int r = 0; r < RPW; ++r) {
@@ -442,6 +574,17 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KER
 // [16384, 2 x 4096] 116.2 -> 98.2 us.
 template <typename InT> constexpr int swiglu_pieces() { return sizeof(InT) == 4 ? 2 : 4; }
 
+// Waves the current GPU holds at once at this kernel's occupancy (8 per SIMD, 4 SIMDs per compute unit).
+static int64_t wave_slots() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus = n;
+    }
+    return (int64_t)cus * 32;
+}
+
 template <typename InT, int CLAMP, int RPW, int TILE>
 static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t stream) {
     // T_ROW, rows per workgroup (= waves), us per call at [8192, 4096] dense / [48128, 4096] with a third of the rows
@@ -462,6 +605,40 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
     // run-time test costs the [8192, 2 x 2048] call 0.2 us
     constexpr bool ROWWISE = TILE == T_ROW || TILE == T_ROWC;
     const bool onecol = ROWWISE && p.tiles_k == 1;
+    if constexpr (TILE == T_ROW && CLAMP != 2 && RPW == 4) {
+        // Finer-grained waves at the end of the launch (see the kernel): the last rows by two-piece waves, 2.2 times the GPU's
+        // wave slots of them but at most 55 % of the rows, and of those the last by one-piece waves, 0.6 times the slots, at
+        // most 15 % of the rows.  For launches of 0.75 to 3.5 times the GPU's wave slots in one-row waves, where it was
+        // measured to pay (bf16, us per call without / with): [6144, 2 x 2048] 11.40 / 11.31, [8192, 2 x 2048] 14.54 / 14.13,
+        // [10240, 2 x 2048] 17.84 / 17.18, [16384, 2 x 2048] 26.92 / 26.50, [8192, 2 x 4096] 26.59 / 26.17, [2048, 2 x 8192]
+        // 14.77 / 14.32, [24576, 2 x 2048] 42.92 / 42.54; smaller and larger launches lose with it ([4096, 2 x 2048] 8.11 / 8.48,
+        // [32768, 2 x 2048] 57.37 / 57.71), and so does a masked batch ([48128, 2 x 2048], a third of the rows padding, 59.9 / 61.8).
+        const int64_t slots = wave_slots(), ppr = p.H / kStripCols, row_waves = (int64_t)p.R * ppr / RPW;
+        const int rs = (int)std::min<int64_t>((int64_t)p.R * 15 / 100, slots * 6 / 10 / ppr) / 4 * 4;
+        const int rm = (int)std::min<int64_t>((int64_t)p.R * 55 / 100, slots * 22 / 10 / ppr) / 4 * 4;
+        const int rb = p.R - rm - rs;
+        const int64_t ym = (int64_t)rm * 2 / waves, ys = (int64_t)rs * 4 / waves, yb = rb / waves;
+        if (full && !p.pos_to_expert && row_waves * 4 >= slots * 3 && row_waves * 2 <= slots * 7 && rs > 0 && p.tiles_k <= 0xFFF &&
+            ym <= 0xFFFF) {
+            const dim3 tgrid = tile_grid(p.tiles_k, (int)(yb + ym + ys));
+            p.nwaves = waves | (p.tiles_k << 4) | ((int)ym << 16);
+            p.tiles_k = (int)yb;
+            p.pos_to_expert = reinterpret_cast<const int32_t *>(static_cast<intptr_t>(p.sf.ld));     // a preloaded place for it
+#define TK_SWIGLU_LAUNCH_TAILED(W_)                                                                                             \
+    do {                                                                                                                        \
+        if (onecol)                                                                                                             \
+            hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, true, false, true, W_>), tgrid, block, 0, stream,     \
+                               TK_SWIGLU_LAUNCH_ARGS(p));                                                                       \
+        else                                                                                                                    \
+            hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, true, false, false, W_>), tgrid, block, 0, stream,    \
+                               TK_SWIGLU_LAUNCH_ARGS(p));                                                                       \
+    } while (0)
+            if (p.pos_to_token_topk) TK_SWIGLU_LAUNCH_TAILED(2);
+            else TK_SWIGLU_LAUNCH_TAILED(1);
+#undef TK_SWIGLU_LAUNCH_TAILED
+            return;
+        }
+    }
 #define TK_SWIGLU_LAUNCH(FULL_, MASK_)                                                                                          \
     do {                                                                                                                        \
         if (onecol)                                                                                                             \

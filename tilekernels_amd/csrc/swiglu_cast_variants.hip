@@ -18,13 +18,15 @@
 //   ahead:n      pieces requested n (1, 2) ahead of the one being evaluated instead of all at once; a piece's scales
 //                are computed and its codes stored before the next piece is waited for
 //   rounds:p     p (1, 2) pieces per wave instead of 4: 4 / p times the waves, in 4 / p occupancy rounds at [8192, 4096]
+//   tail:t       (H = 2048 only) the last t per cent of the rows as four one-piece waves each, launched behind the one-row
+//                waves of the other rows: the work that arrives last is then spread over four times as many SIMDs
 #include "swiglu_math.hpp"
 #include "tk_device.hpp"
 #include "tk_host.hpp"
 
 namespace tk {
 
-enum { V_BASE = 0, V_PKFLOOR = 1, V_WIDEST = 2, V_PRIO = 3, V_PIECESF = 4, V_LATE = 5, V_AHEAD = 6, V_ROUNDS = 7 };
+enum { V_BASE = 0, V_PKFLOOR = 1, V_WIDEST = 2, V_PRIO = 3, V_PIECESF = 4, V_LATE = 5, V_AHEAD = 6, V_ROUNDS = 7, V_TAIL = 8 };
 
 // the eight activations of one lane's piece
 template <bool PKFLOOR> __device__ __forceinline__ void eval_piece(const u32x4 &gw, const u32x4 &uw, float (&v)[8]) {
@@ -167,6 +169,45 @@ __global__ __launch_bounds__(64 * kMaxWideWaves) void swiglu_variant_kernel(cons
     }
 }
 
+// H = 2048: workgroups below `big` hold four rows, one per wave (four pieces each); every later workgroup holds one row,
+// one piece per wave
+__global__ __launch_bounds__(kThreads) void swiglu_tail_kernel(const bf16_t *x, int R, int big, uint8_t *out, float *sf, float floor_) {
+    constexpr int H = 2048, GPS = kStripCols / 128;
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const int wg = blockIdx.x;
+    if (wg < big) {
+        const int row = wg * kWaves + wave;
+        const int col = lane * 8;
+        const bf16_t *xr = x + (int64_t)row * (2 * H) + col;
+        u32x4 gw[4], uw[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            gw[r] = ld_stream16(xr + r * kStripCols);
+            uw[r] = ld_stream16(xr + H + r * kStripCols);
+        }
+        float v[4][8], amax[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            eval_piece<false>(gw[r], uw[r], v[r]);
+            amax[r] = group_allmax<16>(absmax8(v[r]));
+        }
+        RowScales<448, 4, 16> rs;
+        rs.compute(amax, floor_, false, lane);
+        if ((lane & 15) < 4) st_stream4(sf + (int64_t)row * (H / 128) + (lane & 15) * GPS + (lane >> 4), f2u(rs.own[0].sf));
+#pragma unroll
+        for (int r = 0; r < 4; ++r) st_stream8(out + (int64_t)row * H + col + r * kStripCols, convert_piece(v[r], rs.inv[r]));
+    } else {
+        const int row = big * kWaves + (wg - big);
+        const int col = wave * kStripCols + lane * 8;
+        const bf16_t *xr = x + (int64_t)row * (2 * H) + col;
+        const u32x4 gw = ld_stream16(xr), uw = ld_stream16(xr + H);
+        float v[8];
+        eval_piece<false>(gw, uw, v);
+        const float inv = own_scale_store(group_allmax<16>(absmax8(v)), floor_, sf + (int64_t)row * (H / 128), wave * GPS + (lane >> 4), lane);
+        st_stream8(out + (int64_t)row * H + col, convert_piece(v, inv));
+    }
+}
+
 template <int VARIANT, int RPW, int AHEAD = 0>
 static hipError_t launch_variant(const void *x, int R, int H, void *out, void *sf, int waves, int param, hipStream_t stream) {
     const int tiles_k = H / (RPW * kStripCols), tiles_m = (R + waves - 1) / waves;
@@ -211,6 +252,14 @@ extern "C" int tk_swiglu_cast_variant(const void *x, int64_t R, int64_t H, void 
             else if (param == 1) e = launch_variant<V_BASE, 1>(x, r, h, out, sf, kWaves, 0, s);
             else return TK_ERR_BAD_VALUE;
             break;
+        case V_TAIL: {
+            if (h != 2048 || param < 0 || param > 100) return TK_ERR_BAD_VALUE;
+            const int small_rows = (int)((int64_t)r * param / 100) / kWaves * kWaves, big = (r - small_rows) / kWaves;
+            hipLaunchKernelGGL(swiglu_tail_kernel, dim3((unsigned)(big + small_rows)), dim3(kThreads), 0, s, static_cast<const bf16_t *>(x), r,
+                               big, static_cast<uint8_t *>(out), static_cast<float *>(sf), 1e-4f);
+            e = hipGetLastError();
+            break;
+        }
         default: return TK_ERR_BAD_MODE;
     }
     return (int)e;
