@@ -106,6 +106,49 @@ def test_swiglu_fp32_input_tiles(H, with_mask, mode):
     check_fused(got, want, H // 128, packed, f'fp32 H={H}')
 
 
+@pytest.mark.parametrize('clamp', [None, 0.5])
+@pytest.mark.parametrize('rnd', [False, True])
+@pytest.mark.parametrize('with_weights', [False, True])
+@pytest.mark.parametrize('R,H', [(6144, 2048), (3076, 4096), (8192, 2048), (1600, 8192)])
+def test_swiglu_launches_that_end_in_smaller_waves(R, H, with_weights, rnd, clamp):
+    """Unmasked bf16 batches of about one to three times the GPU's wave slots, row-major scales, H a multiple of 2048: the
+    last rows are handled by waves of two pieces and of one piece (a different kernel path with its own argument handling).
+    Rows, weights, clamp and the power-of-two scales must come out as from the one-row waves."""
+    tk = _tk()
+    g = torch.Generator().manual_seed(R + H + int(with_weights))
+    x = (torch.randn((R, 2 * H), generator=g) * 1.5).to(torch.bfloat16)
+    ptt = w = None
+    if with_weights:
+        ptt = torch.randperm(R, generator=g).to(torch.int32)
+        ptt[torch.rand(R, generator=g) < 0.05] = -1                 # rows without a routing slot get weight 0
+        w = torch.rand(((R + 7) // 8, 8), generator=g) + 0.25
+    kw = dict(round_sf=rnd, swiglu_clamp_value=clamp)
+    want = torch_ref.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, ptt, w, None, **kw)
+    got = tk.quant.swiglu_forward_and_per_token_cast(x.cuda(), 'e4m3', 128, None if ptt is None else ptt.cuda(),
+                                                     None if w is None else w.cuda(), None, **kw)
+    check_fused(got, want, H // 128, False, f'R={R} H={H}')
+
+
+def test_swiglu_smaller_waves_with_padded_scale_rows():
+    """Through the C ABI: scale rows with a leading dimension larger than the number of groups (the tail waves take it from a
+    different kernel argument than the one-row waves)."""
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    R, H, ld = 8192, 2048, 24
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn((R, 2 * H), generator=g).to(torch.bfloat16)
+    want_codes, want_sf = torch_ref.swiglu_forward_and_per_token_cast(x, 'e4m3', 128)
+    xg = x.cuda()
+    codes = torch.empty((R, H), dtype=torch.uint8, device='cuda')
+    sf = torch.full((R, ld), -1.0, dtype=torch.float32, device='cuda')
+    rc = lib.tk_swiglu_per_token_cast(xg.data_ptr(), _ffi.TK_BF16, R, H, codes.data_ptr(), sf.data_ptr(), ld, 128, _ffi.TK_SF_ROW_F32, 0, -1.0,
+                                      0, 0, 0, 0, 0, 0.0, 0, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    check_fused((codes.view(torch.float8_e4m3fn), sf[:, :16].contiguous()), (want_codes, want_sf), 16, False, 'padded scale rows')
+    assert torch.all(sf[:, 16:].cpu() == -1.0)
+
+
 def test_swiglu_fp32_input_and_custom_floor():
     tk = _tk()
     x = torch.randn((50, 512)) * 3
