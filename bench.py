@@ -48,7 +48,7 @@ LLC_BYTES = 256 << 20
 # HBM bytes per launch from rocprofv3 counter runs of this script (FETCH_SIZE and WRITE_SIZE, each
 # scaled by what the same counter reads for the 256 MiB copy of --copy-calibration); the summaries
 # are kept under profiles/.  None where no counter run was made.
-MEASURED_TRAFFIC_BYTES = {1: 89.03e6, 2: 44.14e6, 3: 84.48e6, 4: 371.82e6, 5: 297.31e6}
+MEASURED_TRAFFIC_BYTES = {1: 89.04e6, 2: 44.14e6, 3: 84.59e6, 4: 371.83e6, 5: 297.31e6}
 
 WORKLOADS = {
     1: 'per_token_cast e4m3 1x128, bf16 [4096,7168]',
@@ -176,24 +176,33 @@ def preheat(w: 'Workload', ms: float) -> float:
 
 
 def time_gpu(w: 'Workload', steps: int, warmup: int):
-    """Returns (wall seconds for `steps` launches, HIP-event microseconds per launch over the same
-    timed region, list of single-launch durations from per-launch event pairs)."""
+    """Returns (wall seconds for `steps` launches, HIP-event microseconds per launch, the same with the first launch
+    left in, list of single-launch durations from per-launch event pairs).
+
+    The timed region starts on an idle GPU (it follows a synchronisation), and the first launch needs a few
+    microseconds to get there that are no part of any kernel's duration (a kernel trace does not show them either).
+    The per-launch figure is therefore the period of the launches behind the first: an event goes into the stream
+    right behind the first launch, and the time from there to the end of the region is divided by steps - 1.  The wall
+    clock covers all `steps` launches."""
     for i in range(warmup):
         w.launch(i)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0, ef, e1 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
     todo = [w.calls[i % w.nsets] for i in range(steps)]
     e0.record()          # torch's current stream is the stream the launches go to
     t0 = time.perf_counter()
-    for fn, call_args in todo:
+    for n, (fn, call_args) in enumerate(todo):
         if fn(*call_args) != 0:
             raise RuntimeError('launch failed')
+        if n == 0:
+            ef.record()
     e1.record()
     while not e1.query():     # the end of the region is seen by polling: a blocking wait wakes up tens of microseconds late
         pass
     wall = time.perf_counter() - t0
     torch.cuda.synchronize()
-    region_us = e0.elapsed_time(e1) * 1e3 / steps
+    region_all_us = e0.elapsed_time(e1) * 1e3 / steps
+    region_us = ef.elapsed_time(e1) * 1e3 / (steps - 1) if steps >= 4 else region_all_us
     # single launches: one event pair around each (adds the cost of the two event records)
     n = min(steps, 200)
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
@@ -203,7 +212,7 @@ def time_gpu(w: 'Workload', steps: int, warmup: int):
         ev[i][1].record()
     torch.cuda.synchronize()
     per = [a.elapsed_time(b) * 1e3 for a, b in ev]
-    return wall, region_us, per
+    return wall, region_us, region_all_us, per
 
 
 def _event_time_us(fn, n: int) -> float:
@@ -539,7 +548,7 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_str
                  cpu_budget_s: float = 12.0, with_reference: bool = True, traffic: dict = None):
     w = Workload(cfg)
     heated = preheat(w, preheat_ms)
-    wall, kern_us, per = time_gpu(w, steps, warmup)
+    wall, kern_us, kern_all_us, per = time_gpu(w, steps, warmup)
     ms_per_step = wall / steps * 1e3
     value = w.bytes / (wall / steps) / 1e9
     achieved = w.bytes / (kern_us * 1e-6) / 1e9
@@ -557,7 +566,11 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_str
                      'traffic': float(traffic['bytes']) if traffic and 'bytes' in traffic else MEASURED_TRAFFIC_BYTES[cfg],
                      'traffic_source': ('rocprofv3 FETCH_SIZE and WRITE_SIZE runs started by this run' if traffic and 'bytes' in traffic
                                         else 'earlier rocprofv3 counter runs of this script (profiles/)'),
-                     'kernel_us': round(kern_us, 3), 'timing': f'HIP events around the {steps} timed launches / {steps}',
+                     'kernel_us': round(kern_us, 3),
+                     'timing': (f'HIP events: from behind the first of the {steps} timed launches to the end of the region / {steps - 1} '
+                                '(the region starts on an idle GPU; what the first launch takes to get there is no kernel time)'
+                                if steps >= 4 else f'HIP events around the {steps} timed launches / {steps}'),
+                     'kernel_us_first_launch_included': round(kern_all_us, 3),
                      'single_launch_us_median': round(statistics.median(per), 3), 'single_launch_us_min': round(min(per), 3)},
     }
     if with_reference:
