@@ -262,6 +262,20 @@ def same_traffic_reference(w: 'Workload', steps: int):
     us = _event_time_us(floor, n)
     res['traffic_only_kernel'] = {'what': 'tk_stream_floor: the loads and stores of this operator, no arithmetic',
                                   'us_per_call': round(us, 3), 'pct_of_hbm_peak': round(w.bytes / us / 1e3 / HBM_PEAK_GBS * 100, 2)}
+    if w.cfg == 3:
+        # the same traffic in the launch shape the operator uses at this size: the last 15 % of the rows by one-piece waves,
+        # the 55 % before them by two-piece waves (tk_swiglu_per_token_cast, launches of about one to three occupancy rounds)
+        r1, r2 = rows * 15 // 100 // 4 * 4, rows * 55 // 100 // 4 * 4
+
+        def floor_tailed(i):
+            k = i % w.nsets
+            rc = w.lib.tk_stream_floor_tailed(w.x[k].data_ptr(), rows, cols, 1, w.out[k].data_ptr(), w.sf[k].data_ptr(), r2, r1, stream)
+            if rc != 0:
+                raise RuntimeError(f'tk_stream_floor_tailed failed with status {rc}')
+        us = _event_time_us(floor_tailed, n)
+        res['traffic_only_kernel_smaller_waves_at_the_end'] = {
+            'what': f'tk_stream_floor_tailed: the same loads and stores, the last {r1} rows by one-piece and the {r2} before them by two-piece waves',
+            'us_per_call': round(us, 3), 'pct_of_hbm_peak': round(w.bytes / us / 1e3 / HBM_PEAK_GBS * 100, 2)}
     us = _event_time_us(stock, n)
     moved = w.bytes - (0 if w.cfg == 2 else w.sf[0].numel() * w.sf[0].element_size())      # the stock kernel writes no scales
     res['stock_torch_kernel'] = {'what': 'torch.gt into a bool tensor of the output shape (same bytes per element, no scales)',

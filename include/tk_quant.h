@@ -344,6 +344,16 @@ int tk_stream_floor_timeline(const void *x, int64_t rows, int64_t cols, int two_
 int64_t tk_stream_floor_stamp_words(int64_t rows, int64_t cols);
 
 /*
+ * tk_stream_floor_tailed: the traffic-only kernel on a launch that ends in smaller waves, as tk_swiglu_per_token_cast
+ * arranges its launches of about one to three occupancy rounds (measurement aid, no counterpart in the reference): the
+ * last rows_one rows are read and written by four waves of one 512-column piece each, the rows_two rows before them by
+ * two waves of two pieces, the others by one wave of four pieces per 2048 columns.  Same output as tk_stream_floor.
+ *   requirements cols % 2048 == 0; rows, rows_two, rows_one multiples of 4; x 16-byte, out 8-byte aligned
+ */
+int tk_stream_floor_tailed(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, int64_t rows_two,
+                           int64_t rows_one, void *stream);
+
+/*
  * tk_stream_floor_flat: the traffic-only kernel for any ratio of bytes read to bytes written (measurement aid, no
  * counterpart in the reference; bench_ops.py times it beside the operators around the path).  The input is a flat range of
  * in_bytes bytes; a lane reads in_bytes_per_lane (16, 8 or 4) bytes per piece of 64 lanes and writes out_bytes_per_lane

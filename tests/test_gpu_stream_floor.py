@@ -43,6 +43,33 @@ def test_stream_floor_reads_and_writes_everything(rows, cols, two):
     assert np.array_equal(sf.cpu().numpy().view(np.uint32), want_sf)
 
 
+@pytest.mark.parametrize('rows,cols,two,r2,r1', [(64, 2048, True, 24, 12), (40, 4096, False, 20, 8), (16, 2048, True, 0, 16), (16, 2048, True, 16, 0), (8, 6144, True, 0, 0)])
+def test_stream_floor_with_smaller_waves_at_the_end_writes_the_same(rows, cols, two, r2, r1):
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    width = cols * (2 if two else 1)
+    xd = torch.randint(-2 ** 15, 2 ** 15, (rows, width), dtype=torch.int16, device='cuda')
+    stream = torch.cuda.current_stream().cuda_stream
+    out = [torch.full((rows, cols), 0xAB, dtype=torch.uint8, device='cuda') for _ in range(2)]
+    assert lib.tk_stream_floor(xd.data_ptr(), rows, cols, int(two), out[0].data_ptr(), 0, stream) == 0
+    sf = torch.full((rows, cols // 128), -1, dtype=torch.int32, device='cuda')
+    assert lib.tk_stream_floor_tailed(xd.data_ptr(), rows, cols, int(two), out[1].data_ptr(), sf.data_ptr(), r2, r1, stream) == 0
+    assert lib.tk_stream_floor_tailed(xd.data_ptr(), rows, cols, int(two), out[1].data_ptr(), sf.data_ptr(), rows, 4, stream) != 0   # more than there are
+    torch.cuda.synchronize()
+    assert torch.equal(out[0], out[1])
+    # a scale word is the XOR of the first word its lane loaded of each of its wave's pieces: with one piece per wave that
+    # is the first word of the group's own piece at lane 16 * g + (piece mod 1) = 16 * g
+    w = xd.cpu().numpy().view(np.uint32).reshape(rows, width // 2)
+    if two:
+        w = w[:, : cols // 2] ^ w[:, cols // 2:]
+    got = sf.cpu().numpy().view(np.uint32)
+    for row in range(rows - r1, rows):
+        for piece in range(cols // 512):
+            for g in range(4):
+                assert got[row, piece * 4 + g] == w[row, (piece * 512 + 16 * g * 8) // 2]
+    assert not bool((sf == -1).any())
+
+
 def test_stream_floor_rejects_bad_shapes():
     from tilekernels_amd import _ffi
     lib = _ffi.load()

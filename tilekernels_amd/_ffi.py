@@ -52,6 +52,7 @@ SIGNATURES = {
     'tk_stream_floor': (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _vp]),
     'tk_stream_floor_timeline': (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _vp, _vp]),
     'tk_stream_floor_stamp_words': (_i64, [_i64, _i64]),
+    'tk_stream_floor_tailed': (_i32, [_vp, _i64, _i64, _i32, _vp, _vp, _i64, _i64, _vp]),
     'tk_stream_floor_flat': (_i32, [_vp, _i64, _i32, _vp, _i32, _i32, _vp]),
     'tk_swiglu_cast_variant': (_i32, [_vp, _i64, _i64, _vp, _vp, _i32, _i32, _vp]),
     'tk_strerror': (ctypes.c_char_p, [_i32]),

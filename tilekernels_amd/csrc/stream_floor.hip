@@ -68,6 +68,48 @@ __global__ __launch_bounds__(kThreads) void stream_floor_kernel(const bf16_t *x,
     }
 }
 
+// The traffic of a launch that ends in smaller waves, as tk_swiglu_per_token_cast arranges its launches of about one to
+// three occupancy rounds: row tiles [0, yb) are four rows of four-piece waves, the next ym workgroups hold two rows of
+// two-piece waves, the rest one row of one-piece waves.  Same loads, stores and scale words as stream_floor_kernel.
+template <bool TWO>
+__global__ __launch_bounds__(kThreads) void stream_floor_tailed_kernel(const bf16_t *x, int rows, int cols, uint8_t *out, uint32_t *sf,
+                                                                       int tiles_k, int yb, int ym) {
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const int y = tile_grid_row(tiles_k == 1), strip0 = tile_grid_col(tiles_k == 1) * 4;
+    int row, strip, np;
+    if (y < yb) {
+        row = y * kWaves + wave; strip = strip0; np = 4;
+    } else if (y - yb < ym) {
+        const int sub = (y - yb) * kWaves + wave;
+        row = yb * kWaves + (sub >> 1); strip = strip0 + (sub & 1) * 2; np = 2;
+    } else {
+        const int sub = (y - yb - ym) * kWaves + wave;
+        row = yb * kWaves + ym * 2 + (sub >> 2); strip = strip0 + (sub & 3); np = 1;
+    }
+    if (row >= rows) return;
+    const int col = strip * kStripCols + lane * 8;
+    const int64_t ld = (int64_t)cols * (TWO ? 2 : 1);
+    const bf16_t *src = x + row * ld + col;
+    u32x4 a[4], b[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (r < np) {      // wave-uniform
+            a[r] = ld_stream16(src + r * kStripCols);
+            b[r] = TWO ? ld_stream16(src + cols + r * kStripCols) : u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+    uint32_t fold = 0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (r < np) {
+            const u32x4 v = a[r] ^ b[r];
+            st_stream8(out + (int64_t)row * cols + col + r * kStripCols, u32x2{v.x ^ v.z, v.y ^ v.w});
+            fold ^= v.x;
+        }
+    }
+    if (sf != nullptr && (lane & 15) < np) st_stream4(sf + (int64_t)row * (cols / 128) + (strip + (lane & 15)) * 4 + (lane >> 4), fold);
+}
+
 // The same idea for any ratio of bytes read to bytes written: a lane reads IN (16, 8 or 4) bytes per piece and writes OUT
 // (16, 8, 4 or 0) bytes per piece, a piece being 64 lanes side by side; a wave takes PIECES consecutive pieces, all loads
 // issued before the first store.  Input and output are flat byte ranges.
@@ -181,6 +223,28 @@ static int stream_floor_launch(const void *x, int64_t rows, int64_t cols, int tw
 
 extern "C" int tk_stream_floor(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, void *stream) {
     return stream_floor_launch(x, rows, cols, two_halves, out, sf, nullptr, false, stream);
+}
+
+extern "C" int tk_stream_floor_tailed(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, int64_t rows_two,
+                                      int64_t rows_one, void *stream) {
+    if (rows < 0 || cols <= 0 || cols % 2048 != 0 || rows % 4 != 0 || rows_two < 0 || rows_one < 0 || rows_two % 4 != 0 || rows_one % 4 != 0 ||
+        rows_two + rows_one > rows)
+        return TK_ERR_BAD_SHAPE;
+    if (rows > INT32_MAX / 8 || cols > (INT32_MAX - 1024) / 2) return TK_ERR_TOO_LARGE;
+    if (rows == 0) return TK_OK;
+    if (!x || !out) return TK_ERR_NULL_POINTER;
+    if (!aligned_to(x, 16) || !aligned_to(out, 8) || !aligned_to(sf, 4)) return TK_ERR_MISALIGNED;
+    const int tiles_k = (int)(cols / (4 * kStripCols));
+    const int yb = (int)((rows - rows_two - rows_one) / kWaves), ym = (int)(rows_two * 2 / kWaves), ys = (int)(rows_one * 4 / kWaves);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid = tile_grid(tiles_k, yb + ym + ys);
+    if (two_halves)
+        hipLaunchKernelGGL(stream_floor_tailed_kernel<true>, grid, dim3(kThreads), 0, s, static_cast<const bf16_t *>(x), (int)rows, (int)cols,
+                           static_cast<uint8_t *>(out), static_cast<uint32_t *>(sf), tiles_k, yb, ym);
+    else
+        hipLaunchKernelGGL(stream_floor_tailed_kernel<false>, grid, dim3(kThreads), 0, s, static_cast<const bf16_t *>(x), (int)rows, (int)cols,
+                           static_cast<uint8_t *>(out), static_cast<uint32_t *>(sf), tiles_k, yb, ym);
+    return (int)hipGetLastError();
 }
 
 extern "C" int64_t tk_stream_floor_stamp_words(int64_t rows, int64_t cols) {
