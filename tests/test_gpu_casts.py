@@ -267,6 +267,22 @@ def test_cast_back(M, K, block, fmt, mode, out_fmt):
         assert_same(tk.quant.per_token_cast_back((q[0].cuda(), _to_gpu_like(q[1])), out_fmt, block[1]), want, 'per-token back')
 
 
+@pytest.mark.parametrize('out_fmt', ['bf16', 'fp32'])
+@pytest.mark.parametrize('mode', [(False, False, False), (True, False, False), (True, True, True)], ids=_mode_id)
+@pytest.mark.parametrize('fmt', ['e4m3', 'e2m1'])
+@pytest.mark.parametrize('M,K,block', [(257, 512, (128, 1)), (130, 192, (32, 2)), (64, 1088, (128, 4)), (300, 64, (1, 4)), (129, 2048, (128, 1))])
+def test_cast_back_with_scale_blocks_narrower_than_a_lane(M, K, block, fmt, mode, out_fmt):
+    """Scale blocks of 1, 2 or 4 columns (the per-channel 128 x 1 scales among them): a lane's 8 codes then carry 8, 4 or 2
+    different scales, which a kernel of its own fetches; both code formats, every scale layout."""
+    tk = _tk()
+    col, rnd, packed = mode
+    x = _rand((M, K), torch.bfloat16)
+    q = torch_ref.cast(x, fmt, block, use_tma_aligned_col_major_sf=col, round_sf=rnd, use_packed_ue8m0=packed)
+    want = torch_ref.cast_back(q, out_fmt, block)
+    got = tk.quant.cast_back((q[0].cuda(), _to_gpu_like(q[1])), out_fmt, block)
+    assert_same(got, want, 'dequantised')
+
+
 def test_cast_then_cast_back_round_trip_on_device():
     tk = _tk()
     x = _rand((512, 4096), torch.bfloat16).cuda()
