@@ -9,6 +9,8 @@
 //
 // Reference semantics: tile_kernels/quant/swiglu_forward_and_per_token_cast_kernel.py:61-170,
 // tile_kernels/torch/swiglu.py:62-86.
+#include <stddef.h>
+
 #include <algorithm>
 
 #include "swiglu_math.hpp"
@@ -86,6 +88,8 @@ struct SwigluKernargs {
     const void *x; const int32_t *pe; int R, H, nwaves, tiles_k; uint8_t *out; void *sf; float floor_; int round_sf;
     SwigluLateKernargs late;
 };
+static_assert(offsetof(SwigluKernargs, late) == 56 && offsetof(SwigluLateKernargs, ptt) == 16 && offsetof(SwigluLateKernargs, nw) == 40,
+              "the mirror of the argument segment follows TK_SWIGLU_KERNEL_ARGS: 14 preloaded dwords, then the later arguments");
 
 // The arguments beyond the preloaded ones that the row-wise waves use after their vector loads, read from the argument
 // segment here and now.  A kernel whose code paths part before the loads names these arguments nowhere else: named, their
