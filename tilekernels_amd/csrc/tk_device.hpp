@@ -334,10 +334,46 @@ template <int QMAX> __device__ __forceinline__ float div_by_qmax(float a) {
     return __builtin_fmaf(__builtin_fmaf(-c, q, a), y, q);
 }
 
+// QMAX / a for a in [2^-60, 2^60]: the instructions of the IEEE division (reciprocal, one refinement of it, the quotient,
+// one refinement, the final residual step) without its operand scaling and its special-case fix-up; on this range
+// v_div_scale_f32 returns its operands unchanged and v_div_fixup_f32 the quotient it is given, so the result is
+// QMAX / a bit for bit (compared on MI355X with the compiler's division for each of the 1006632961 floats of the range,
+// for 448 and for 6, together with the three-instruction a / QMAX above: no difference).
+template <int QMAX> __device__ __forceinline__ float qmax_over_plain(float a) {
+    constexpr float n = (float)QMAX;
+    float r = __builtin_amdgcn_rcpf(a);
+    r = __builtin_fmaf(__builtin_fmaf(-a, r, 1.0f), r, r);
+    float q = n * r;
+    q = __builtin_fmaf(__builtin_fmaf(-a, q, n), r, q);
+    return __builtin_fmaf(__builtin_fmaf(-a, q, n), r, q);
+}
+
 template <int QMAX> __device__ __forceinline__ Scale make_scale(float amax, float floor_, bool round_sf) {
     const float a = __builtin_fmaxf(amax, floor_);
-    const float s = div_by_qmax<QMAX>(a);
     Scale r;
+    if constexpr (QMAX == 448 || QMAX == 6) {
+        // Maxima between 2^-60 and 2^60 in every lane (what any real tensor gives): both divisions in their short forms, chosen
+        // by one branch for the wave, so the long forms cost nothing where they are not needed
+        const bool plain = f2u(a) - 0x21800000u <= 0x5D800000u - 0x21800000u;
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(!plain) == 0, 1)) {
+            constexpr float c = (float)QMAX;
+            constexpr float y = 1.0f / c;
+            const float q = a * y;
+            const float s = __builtin_fmaf(__builtin_fmaf(-c, q, a), y, q);
+            if (!round_sf) {
+                r.sf = s;
+                r.inv = qmax_over_plain<QMAX>(a);
+                r.e8 = f2u(s) >> 23;
+            } else {
+                const uint32_t b = (f2u(s) + 0x007FFFFFu) & 0x7F800000u;
+                r.sf = u2f(b);
+                r.e8 = b >> 23;
+                r.inv = u2f((254u << 23) - b);      // the exponent of s is between 58 and 179 here
+            }
+            return r;
+        }
+    }
+    const float s = div_by_qmax<QMAX>(a);
     if (!round_sf) {
         r.sf = s;
         r.inv = f2u(s) == 0u ? 0.0f : (float)QMAX / a;
@@ -410,9 +446,11 @@ template <bool CLAMP> __device__ __forceinline__ u32x2 pack_e4m3x8(const float (
     float c[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) c[i] = CLAMP ? __builtin_amdgcn_fmed3f(q[i], -448.0f, 448.0f) : q[i];
-    int lo = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], 0, false);
+    // (the first conversion of a dword fills its low half and keeps the rest of its third operand, which the second one
+    // overwrites: any register that is at hand serves, and a zero would have to be made first)
+    int lo = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], (int)f2u(c[0]), false);
     lo = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], lo, true);
-    int hi = __builtin_amdgcn_cvt_pk_fp8_f32(c[4], c[5], 0, false);
+    int hi = __builtin_amdgcn_cvt_pk_fp8_f32(c[4], c[5], (int)f2u(c[4]), false);
     hi = __builtin_amdgcn_cvt_pk_fp8_f32(c[6], c[7], hi, true);
     return u32x2{(uint32_t)lo, (uint32_t)hi};
 }
