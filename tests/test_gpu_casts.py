@@ -171,6 +171,38 @@ def test_device_e2m1_conversion_at_every_boundary():
     assert_same(got, torch_ref.cast(x, 'e2m1', (1, 32), sf=ones), 'e2m1 codes')
 
 
+@pytest.mark.parametrize('rnd', [False, True], ids=['exact_sf', 'round_sf'])
+@pytest.mark.parametrize('fmt,N', [('e4m3', 128), ('e2m1', 32), ('e4m3', 32)])
+def test_group_maxima_over_the_whole_exponent_range(fmt, N, rnd):
+    """Group maxima from 2^-126 to 2^126: the scale divisions take their short forms between 2^-60 and 2^60 and the
+    general ones outside, decided per wave, so groups of both kinds share waves here; codes and scales stay bit-exact."""
+    tk = _tk()
+    g = torch.Generator().manual_seed(11)
+    K = 2048
+    exps = torch.arange(-126, 127)
+    rows = []
+    for rep in range(3):
+        k = exps[torch.randint(0, exps.numel(), (12, K // N), generator=g)]
+        x = torch.randn((12, K), generator=g).clamp(-3, 3) * torch.exp2(k.float() - 2).repeat_interleave(N, dim=1)
+        rows.append(x)
+    # rows that stay inside the short-form range, rows that stay outside, and mixed ones (above)
+    rows.append(torch.randn((8, K), generator=g) * 2.0 ** 40)
+    rows.append(torch.randn((8, K), generator=g) * 2.0 ** -70)
+    rows.append(torch.randn((8, K), generator=g).clamp(-3, 3) * 2.0 ** 100)
+    x = torch.cat(rows)
+    assert torch.isfinite(x).all()
+    codes, sf = tk.quant.per_token_cast(x.cuda(), fmt, N, round_sf=rnd)
+    codes_ref, sf_ref = torch_ref.cast(x, fmt, (1, N), round_sf=rnd)
+    assert_same(sf, sf_ref, 'sf')
+    assert_same(codes, codes_ref, 'codes')
+    if N == 128 or fmt == 'e2m1':
+        xb = x[: x.shape[0] // 128 * 128] if x.shape[0] >= 128 else torch.cat([x] * 4)[:128]
+        cb, sb = tk.quant.per_block_cast(xb.cuda(), fmt, (N, N) if N == 128 else (32, 32), round_sf=rnd)
+        cbr, sbr = torch_ref.cast(xb, fmt, (N, N) if N == 128 else (32, 32), round_sf=rnd)
+        assert_same(sb, sbr, 'block sf')
+        assert_same(cb, cbr, 'block codes')
+
+
 def test_empty_inputs():
     tk = _tk()
     x = torch.empty((0, 256), dtype=torch.bfloat16)
