@@ -175,6 +175,46 @@ def preheat(w: 'Workload', ms: float) -> float:
     return spent
 
 
+def time_gpu_graph(w: 'Workload', steps: int, warmup: int, chunk: int = 100):
+    """The same launches enqueued by the GPU instead of the host: `chunk` launches on the rotating buffers are captured into
+    one HIP graph and the graph is replayed until `steps` launches have run.  Under a profiler the host needs longer per
+    launch than the kernel takes, the GPU idles between launches and the profiler's durations are those of a GPU whose
+    clocks have dropped; replays keep the launches back to back.  Returns what time_gpu returns (the per-launch figure is
+    the whole region over its launches; the first replay runs untimed)."""
+    chunk = max(w.nsets, min(chunk, steps) // w.nsets * w.nsets)      # whole turns of the buffer sets
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        for i in range(max(warmup, w.nsets)):
+            w.launch(i, side.cuda_stream)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(chunk):
+                w.launch(i, side.cuda_stream)
+        replays = max(1, -(-steps // chunk))
+        graph.replay()
+        side.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        t0 = time.perf_counter()
+        for _ in range(replays):
+            graph.replay()
+        e1.record()
+        while not e1.query():
+            pass
+        wall = (time.perf_counter() - t0) * steps / (replays * chunk)
+        us = e0.elapsed_time(e1) * 1e3 / (replays * chunk)
+    torch.cuda.synchronize()
+    n = min(steps, 200)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for i in range(n):
+        ev[i][0].record()
+        w.launch(i)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    return wall, us, us, [a.elapsed_time(b) * 1e3 for a, b in ev]
+
+
 def time_gpu(w: 'Workload', steps: int, warmup: int):
     """Returns (wall seconds for `steps` launches, HIP-event microseconds per launch, the same with the first launch
     left in, list of single-launch durations from per-launch event pairs).
@@ -559,10 +599,10 @@ def cpu_baseline(w: Workload, budget_s: float = 12.0, min_runs: int = 3):
 
 
 def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_streams: bool = True, preheat_ms: float = 40.0,
-                 cpu_budget_s: float = 12.0, with_reference: bool = True, traffic: dict = None):
+                 cpu_budget_s: float = 12.0, with_reference: bool = True, traffic: dict = None, graph: bool = False):
     w = Workload(cfg)
     heated = preheat(w, preheat_ms)
-    wall, kern_us, kern_all_us, per = time_gpu(w, steps, warmup)
+    wall, kern_us, kern_all_us, per = time_gpu_graph(w, steps, warmup) if graph else time_gpu(w, steps, warmup)
     ms_per_step = wall / steps * 1e3
     value = w.bytes / (wall / steps) / 1e9
     achieved = w.bytes / (kern_us * 1e-6) / 1e9
@@ -581,7 +621,8 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_str
                      'traffic_source': ('rocprofv3 FETCH_SIZE and WRITE_SIZE runs started by this run' if traffic and 'bytes' in traffic
                                         else 'earlier rocprofv3 counter runs of this script (profiles/)'),
                      'kernel_us': round(kern_us, 3),
-                     'timing': (f'HIP events: from behind the first of the {steps} timed launches to the end of the region / {steps - 1} '
+                     'timing': ('HIP events around replays of a HIP graph of launches on the rotating buffers (about 100 per replay), per launch' if graph else
+                                f'HIP events: from behind the first of the {steps} timed launches to the end of the region / {steps - 1} '
                                 '(the region starts on an idle GPU; what the first launch takes to get there is no kernel time)'
                                 if steps >= 4 else f'HIP events around the {steps} timed launches / {steps}'),
                      'kernel_us_first_launch_included': round(kern_all_us, 3),
@@ -649,6 +690,9 @@ def main():
     ap.add_argument('--variant', type=str, default=None,
                     help='instead of the benchmark, time alternative structures of the headline kernel against the product: a comma-separated '
                          f'list of {", ".join(VARIANTS)}, each optionally with ":<parameter>" (see csrc/swiglu_cast_variants.hip)')
+    ap.add_argument('--graph', action='store_true',
+                    help='enqueue the timed launches of --config from a HIP graph (100 launches per replay) instead of from the host: '
+                         'for runs under a profiler, where the host is slower than the kernel')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run plain device copies of known size (reference kernel for hardware-counter runs)')
     args = ap.parse_args()
@@ -676,7 +720,8 @@ def main():
     if not torch.cuda.is_available():
         sys.exit('bench.py needs a GPU')
     two = not args.single_stream_only
-    line = bench_config(args.config, args.steps, args.warmup, not args.no_cpu, two, args.preheat_ms, 12.0, two, traffic.get(args.config))
+    line = bench_config(args.config, args.steps, args.warmup, not args.no_cpu, two, args.preheat_ms, 12.0, two, traffic.get(args.config),
+                        args.graph)
     if traffic:
         line['traffic_measurement'] = {str(c): t for c, t in traffic.items()}
     if not args.only:
