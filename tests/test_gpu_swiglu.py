@@ -109,11 +109,15 @@ def test_swiglu_fp32_input_tiles(H, with_mask, mode):
 @pytest.mark.parametrize('clamp', [None, 0.5])
 @pytest.mark.parametrize('rnd', [False, True])
 @pytest.mark.parametrize('with_weights', [False, True])
+@pytest.mark.parametrize('layout', ['row', 'col', 'packed'])
 @pytest.mark.parametrize('R,H', [(6144, 2048), (3076, 4096), (8192, 2048), (1600, 8192)])
-def test_swiglu_launches_that_end_in_smaller_waves(R, H, with_weights, rnd, clamp):
-    """Unmasked bf16 batches of about one to three times the GPU's wave slots, row-major scales, H a multiple of 2048: the
-    last rows are handled by waves of two pieces and of one piece (a different kernel path with its own argument handling).
+def test_swiglu_launches_that_end_in_smaller_waves(R, H, layout, with_weights, rnd, clamp):
+    """Unmasked bf16 batches of about one to three times the GPU's wave slots, H a multiple of 2048: the last rows are
+    handled by waves of two pieces and of one piece (a different kernel path with its own argument handling; with the
+    column-major layouts the four waves of a workgroup take four rows of the same pieces and store their scales together).
     Rows, weights, clamp and the power-of-two scales must come out as from the one-row waves."""
+    if layout == 'packed' and not rnd:
+        pytest.skip('packed scales are powers of two')
     tk = _tk()
     g = torch.Generator().manual_seed(R + H + int(with_weights))
     x = (torch.randn((R, 2 * H), generator=g) * 1.5).to(torch.bfloat16)
@@ -122,11 +126,11 @@ def test_swiglu_launches_that_end_in_smaller_waves(R, H, with_weights, rnd, clam
         ptt = torch.randperm(R, generator=g).to(torch.int32)
         ptt[torch.rand(R, generator=g) < 0.05] = -1                 # rows without a routing slot get weight 0
         w = torch.rand(((R + 7) // 8, 8), generator=g) + 0.25
-    kw = dict(round_sf=rnd, swiglu_clamp_value=clamp)
+    kw = dict(round_sf=rnd, swiglu_clamp_value=clamp, use_tma_aligned_col_major_sf=layout != 'row', use_packed_ue8m0=layout == 'packed')
     want = torch_ref.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, ptt, w, None, **kw)
     got = tk.quant.swiglu_forward_and_per_token_cast(x.cuda(), 'e4m3', 128, None if ptt is None else ptt.cuda(),
                                                      None if w is None else w.cuda(), None, **kw)
-    check_fused(got, want, H // 128, False, f'R={R} H={H}')
+    check_fused(got, want, H // 128, layout == 'packed', f'R={R} H={H} {layout}')
 
 
 def test_swiglu_smaller_waves_with_padded_scale_rows():

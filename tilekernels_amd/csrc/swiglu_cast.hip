@@ -100,11 +100,15 @@ static_assert(offsetof(SwigluKernargs, late) == 56 && offsetof(SwigluLateKernarg
 // (bf16 [8192, 2 x 2048]: 14.7 us with the routing arguments looked at by every wave, 14.3 us without), so only what the
 // variant at hand uses is fetched: the clamp value, the routing list with its weights and their count.  (The leading
 // dimension of the scales, which every wave needs, travels in a preloaded place: see the launch code.)
-__device__ __forceinline__ void fetch_late_arguments(SwigluParams &p, bool with_clamp, bool with_weights) {
+__device__ __forceinline__ void fetch_late_arguments(SwigluParams &p, bool with_clamp, bool with_weights, bool with_layout = false) {
     uintptr_t ka = (uintptr_t)__builtin_amdgcn_kernarg_segment_ptr();
     asm volatile("" : "+s"(ka) : : "memory");      // stays behind the loads issued before it
     const SwigluLateKernargs *k = &reinterpret_cast<const SwigluKernargs *>(ka)->late;
     if (with_clamp) p.clamp = uniform_load(&k->clamp);
+    if (with_layout) {
+        p.sf.layout = uniform_load(&k->sf_layout);
+        p.sf.nk = uniform_load(&k->nk);
+    }
     if (with_weights) {
         p.pos_to_token_topk = uniform_load(&k->ptt);
         p.topk_weights = uniform_load(&k->w);
@@ -120,7 +124,7 @@ __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
 
 // One wave on NP consecutive pieces of one row (row-major scales, which the wave stores itself; no mask; CLAMP 0 or 1):
 // what a wave of a T_ROW tile does, for the finer-grained waves at the end of a launch (see the tiled kernel).
-template <typename InT, int CLAMP, int NP, bool WEIGHTED>
+template <typename InT, int CLAMP, int NP, bool WEIGHTED, bool ROWC = false>
 __device__ __forceinline__ void swiglu_row_wave(SwigluParams p, int row0, int strip) {
     static_assert(CLAMP != 2, "the counting variant loops over tiles");
     static_assert(Raw8<InT>::kXchgBytes == 0, "inputs whose pieces need no exchange between lanes");
@@ -129,13 +133,16 @@ __device__ __forceinline__ void swiglu_row_wave(SwigluParams p, int row0, int st
     const int lane = threadIdx.x & 63, own = lane & 15;
     const int col = strip * kStripCols + lane * 8;
     const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * (2 * (int64_t)p.H) + col;
+    // column-major layouts: the workgroup's four waves hold four consecutive rows of the same pieces; their scales meet in
+    // LDS and leave as runs along the rows
+    __shared__ uint32_t stage[ROWC ? kWaves : 1][ROWC ? NP * GPS : 1];
     Raw8<InT> rg[NP], ru[NP];
 #pragma unroll
     for (int r = 0; r < NP; ++r) {
         rg[r].load(x + r * kStripCols);
         ru[r].load(x + r * kStripCols + p.H);
     }
-    fetch_late_arguments(p, CLAMP != 0, WEIGHTED);
+    fetch_late_arguments(p, CLAMP != 0, WEIGHTED, ROWC);
     const float w = WEIGHTED ? row_weight(p, row0) : 0.0f;
     ClampCounter<CLAMP> clamp;
     float v[NP][8], amax[NP];
@@ -160,11 +167,19 @@ __device__ __forceinline__ void swiglu_row_wave(SwigluParams p, int row0, int st
     // lane j (< A) of a group computed the scale of piece c*A + j; the wave's scales form one run of NP * 4 floats
     if (own < RS::A) {
 #pragma unroll
-        for (int c = 0; c < RS::NC; ++c)
-            st_stream4(reinterpret_cast<float *>(p.sf.base) + (int64_t)row0 * p.sf.ld + (strip + c * RS::A + own) * GPS + (lane >> 4), f2u(rs.own[c].sf));
+        for (int c = 0; c < RS::NC; ++c) {
+            if constexpr (ROWC)
+                stage[wave_id()][(c * RS::A + own) * GPS + (lane >> 4)] = p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
+            else
+                st_stream4(reinterpret_cast<float *>(p.sf.base) + (int64_t)row0 * p.sf.ld + (strip + c * RS::A + own) * GPS + (lane >> 4), f2u(rs.own[c].sf));
+        }
     }
 #pragma unroll
     for (int r = 0; r < NP; ++r) quantise_store8<TK_E4M3, false>(v[r], rs.inv[r], p.out + (int64_t)row0 * p.H, col + r * kStripCols);
+    if constexpr (ROWC) {
+        __syncthreads();
+        sf_store_tile_colmajor<kWaves, NP * GPS>(p.sf, stage, row0 - wave_id(), strip * GPS);
+    }
 }
 
 // Tile shapes (a wave always holds RPW pieces of 512 output columns, each with its gate and its up half):
@@ -194,10 +209,14 @@ enum { T_STACKED = 0, T_ROW = 2, T_ROWC = 3 };
 // 15 % in one-piece waves 14.06 (55 % / 15 % of the rows: 2.2 and 0.6 times the GPU's wave slots).  The arguments pack
 // the run lengths into the two tile-geometry words (see the launch code) so that they arrive preloaded, and the place of
 // the mask pointer (these launches have no mask) carries the leading dimension of the scales.  TAILED: 1 without, 2 with
-// routing weights.
+// routing weights.  T_ROWC tiles end the same way, with the four waves of a workgroup on four consecutive rows of the same
+// two pieces or one piece (swiglu_row_wave<..., ROWC>), so that their scales still leave as runs along the rows; layout
+// and group count of the scales are among the arguments read behind the loads.  bf16, us per call without / with,
+// column-major fp32 scales: [8192, 2 x 2048] 15.39 / 14.74, [4096, 2 x 4096] 15.34 / 14.86, [12288, 2 x 2048] 21.40 / 20.89,
+// [16384, 2 x 2048] 27.53 / 27.13; packed UE8M0: 14.79 / 14.36, 14.70 / 14.47, 21.11 / 20.61, 27.18 / 26.88.
 template <typename InT, int CLAMP, int RPW, int TILE, bool FULL_GRID, bool MASK, bool ONECOL, int TAILED = 0>
 __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
-    static_assert(!TAILED || (TILE == T_ROW && FULL_GRID && !MASK && CLAMP != 2 && RPW == 4), "tail waves: exact unmasked grids of one-row waves of four pieces");
+    static_assert(!TAILED || ((TILE == T_ROW || TILE == T_ROWC) && FULL_GRID && !MASK && CLAMP != 2 && RPW == 4), "tail waves: exact unmasked grids of one-row waves of four pieces");
     if constexpr (TAILED) {
         // a_nwaves: waves per workgroup (bits 0-3), column tiles (4-15), two-piece workgroups (16-31); a_tiles_k: one-row workgroups
         const int yb = a_tiles_k, ym = (int)((unsigned)a_nwaves >> 16);
@@ -210,7 +229,20 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
             const int strip0 = tile_grid_col(one_col) * RPW, wave = wave_id();
             const int rb = yb * p.nwaves;                       // rows done by one-row waves
             int row, strip;
-            if (y - yb < ym) {
+            if constexpr (TILE == T_ROWC) {
+                // four rows per workgroup, one per wave, the same pieces in each
+                if (y - yb < ym) {
+                    const int sub = y - yb;                         // two workgroups per four rows
+                    row = rb + (sub >> 1) * kWaves + wave;
+                    strip = strip0 + (sub & 1) * 2;
+                    swiglu_row_wave<InT, CLAMP, 2, TAILED == 2, true>(p, row, strip);
+                } else {
+                    const int sub = y - yb - ym;                    // four workgroups per four rows
+                    row = rb + ym * 2 + (sub >> 2) * kWaves + wave;
+                    strip = strip0 + (sub & 3);
+                    if (row < p.R) swiglu_row_wave<InT, CLAMP, 1, TAILED == 2, true>(p, row, strip);    // (whole workgroups overhang)
+                }
+            } else if (y - yb < ym) {
                 const int sub = (y - yb) * p.nwaves + wave;     // two waves per row
                 row = rb + (sub >> 1);
                 strip = strip0 + (sub & 1) * 2;
@@ -316,7 +348,7 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
         }
 
         // (in this variant the fetch of the later arguments starts at the head of the kernel, where its paths part)
-        if constexpr (TAILED != 0) fetch_late_arguments(p, CLAMP != 0, TAILED == 2);
+        if constexpr (TAILED != 0) fetch_late_arguments(p, CLAMP != 0, TAILED == 2, TILE == T_ROWC);
         if constexpr (FULL && XB != 0) {
 #pragma unroll
             for (int r = 0; r < RPW; ++r) {
@@ -609,7 +641,7 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
     // run-time test costs the [8192, 2 x 2048] call 0.2 us
     constexpr bool ROWWISE = TILE == T_ROW || TILE == T_ROWC;
     const bool onecol = ROWWISE && p.tiles_k == 1;
-    if constexpr (TILE == T_ROW && CLAMP != 2 && RPW == 4) {
+    if constexpr ((TILE == T_ROW || TILE == T_ROWC) && CLAMP != 2 && RPW == 4) {
         // Finer-grained waves at the end of the launch (see the kernel): the last rows by two-piece waves, 2.2 times the GPU's
         // wave slots of them but at most 55 % of the rows, and of those the last by one-piece waves, 0.6 times the slots, at
         // most 15 % of the rows.  For launches of 0.75 to 3.5 times the GPU's wave slots in one-row waves, where it was
