@@ -107,9 +107,12 @@ __device__ __forceinline__ void st_stream8(void *p, u32x2 v) {
     __hip_atomic_store(reinterpret_cast<uint64_t *>(p), __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_SYSTEM);
 }
-// (the 16-byte form has no builtin with these cache bits)
+// (The 16-byte form has no builtin with these cache bits.  A store of more than 8 bytes must not be followed at once by
+// a VALU instruction that overwrites its data registers; for its own stores the compiler keeps that distance, for an
+// instruction it cannot look into it does not, so the wait state is part of the text.  Without it a loop whose next
+// iteration begins by computing an address in the first data register stored that address instead of the data.)
 __device__ __forceinline__ void st_stream16(void *p, u32x4 v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 0" ::"v"(p), "v"(v) : "memory");
 }
 __device__ __forceinline__ void st_stream4(void *p, uint32_t v) {
     __hip_atomic_store(reinterpret_cast<uint32_t *>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
