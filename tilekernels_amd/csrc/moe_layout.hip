@@ -508,7 +508,9 @@ __global__ __launch_bounds__(kThreads) void reduce_fused_kernel(const typename R
         w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{acc[2], acc[3]}), bf16x2));
         w.z = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{acc[4], acc[5]}), bf16x2));
         w.w = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{acc[6], acc[7]}), bf16x2));
-        __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(out) + idx));
+        // (written through: bf16 [4096, 4096] from top-8 of 256 experts 50.3 -> 49.2 us on MI355X against a non-temporal
+        // store; the stores of most other kernels here lose that way, the expansion 64 -> 110 us)
+        st_stream16(reinterpret_cast<uint16_t *>(out) + idx, w);
     } else if (SPLIT) {
         const u32x2 codes = pack_e4m3x8<false>(acc);
         st_stream4(reinterpret_cast<uint8_t *>(out) + idx, codes.x);
