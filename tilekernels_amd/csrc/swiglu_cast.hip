@@ -122,8 +122,9 @@ __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
     return (pos >= 0 && pos < p.num_weights) ? uniform_load(p.topk_weights + pos) : 0.0f;
 }
 
-// One wave on NP consecutive pieces of one row (row-major scales, which the wave stores itself; no mask; CLAMP 0 or 1):
-// what a wave of a T_ROW tile does, for the finer-grained waves at the end of a launch (see the tiled kernel).
+// One wave on NP consecutive pieces of one row (no mask; CLAMP 0 or 1): what a wave of a T_ROW or T_ROWC tile does, for the
+// finer-grained waves at the end of a launch (see the tiled kernel).  Row-major scales are stored by the wave itself; with
+// ROWC (column-major layouts) the caller's four waves hold rows row0 - wave .. row0 - wave + 3 of the same pieces.
 template <typename InT, int CLAMP, int NP, bool WEIGHTED, bool ROWC = false>
 __device__ __forceinline__ void swiglu_row_wave(SwigluParams p, int row0, int strip) {
     static_assert(CLAMP != 2, "the counting variant loops over tiles");
@@ -197,7 +198,7 @@ __device__ __forceinline__ void swiglu_row_wave(SwigluParams p, int row0, int st
 enum { T_STACKED = 0, T_ROW = 2, T_ROWC = 3 };
 
 // ONECOL: the grid is known to be a single column of tiles (else it is found out at run time)
-// TAILED (T_ROW tiles of four-piece waves, exact grids): the launch ends in finer-grained waves.  The grid's row tiles
+// TAILED (T_ROW and T_ROWC tiles of four-piece waves, exact grids): the launch ends in finer-grained waves.  The grid's row tiles
 // come in three runs: `yb` workgroups of one-row waves as described above, then `ym` workgroups whose waves take two
 // pieces, then workgroups whose waves take one; all cover the rows in order.  The requests of a launch are served
 // roughly in the order they were made, so what arrives last belongs to the last workgroups; with whole rows per wave
