@@ -48,7 +48,7 @@ LLC_BYTES = 256 << 20
 # HBM bytes per launch from rocprofv3 counter runs of this script (FETCH_SIZE and WRITE_SIZE, each
 # scaled by what the same counter reads for the 256 MiB copy of --copy-calibration); the summaries
 # are kept under profiles/.  None where no counter run was made.
-MEASURED_TRAFFIC_BYTES = {1: 89.04e6, 2: 44.14e6, 3: 84.59e6, 4: 371.83e6, 5: 297.31e6}
+MEASURED_TRAFFIC_BYTES = {1: 89.04e6, 2: 44.14e6, 3: 84.61e6, 4: 371.83e6, 5: 297.30e6}
 
 WORKLOADS = {
     1: 'per_token_cast e4m3 1x128, bf16 [4096,7168]',
