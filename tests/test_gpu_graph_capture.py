@@ -69,3 +69,46 @@ def test_moe_chain_replays_from_a_graph():
             assert a.dtype == b.dtype and a.shape == b.shape
             ab, bb = a.contiguous().view(torch.uint8), b.contiguous().view(torch.uint8)
             assert torch.equal(ab, bb), f'seed {seed}: output {i} differs between graph replay and eager run'
+
+
+@pytest.mark.parametrize('layout', ['row', 'packed'])
+def test_swiglu_launch_that_ends_in_smaller_waves_replays_from_a_graph(layout):
+    """The launch shape of dense batches of about one to three times the GPU's wave slots (its smaller waves read part of
+    their arguments from the argument segment behind their loads) under capture: replays on new contents equal eager runs."""
+    import tilekernels_amd as tk
+    R, H = 8192, 2048
+    kw = dict(round_sf=True, use_tma_aligned_col_major_sf=layout == 'packed', use_packed_ue8m0=layout == 'packed')
+    x = torch.empty((R, 2 * H), dtype=torch.bfloat16, device='cuda')
+    ptt = torch.arange(R, dtype=torch.int32, device='cuda')
+    w = torch.empty((R // 8, 8), dtype=torch.float32, device='cuda')
+
+    def run():
+        a = tk.quant.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, **kw)
+        b = tk.quant.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, pos_to_token_topk=ptt, topk_weights=w, swiglu_clamp_value=2.0, **kw)
+        return [a[0], a[1], b[0], b[1]]
+
+    def load(seed):
+        g = torch.Generator().manual_seed(seed)
+        x.copy_(torch.randn((R, 2 * H), generator=g).to(torch.bfloat16))
+        w.copy_(torch.rand((R // 8, 8), generator=g) + 0.5)
+
+    load(0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run()
+    for seed in (1, 2, 3):
+        load(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        _ = (x.float() * 2).sum().item()
+        want = run()
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a.contiguous().view(torch.uint8), b.contiguous().view(torch.uint8)), f'seed {seed}: output {i}'
