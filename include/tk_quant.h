@@ -138,8 +138,10 @@ int tk_check_per_block_cast(const void *x, int x_dtype, int64_t M, int64_t K, co
  *   clamped_count       NULL, or int64[3] incremented by {#g > clamp, #u > clamp, #u < -clamp} over
  *                       the non-padding rows, counted before clamping (needs use_clamp)
  *   max_blocks          with clamped_count: > 0 caps the number of workgroups, which then loop over tiles
- *                       (the reference's num_sms knob for the counting variant; few workgroups touch the
- *                       global counters); <= 0 or without clamped_count: one workgroup per tile
+ *                       (the reference's num_sms knob for the counting variant: every workgroup that clamped
+ *                       anything sends one atomic request to the counters, and requests to one line are served
+ *                       one at a time; the Python wrapper passes 8 per compute unit); <= 0 or without
+ *                       clamped_count: one workgroup per tile
  *   requirements        H % 128 == 0; group == 128, or group == H with TK_SF_ROW_F32; x 16-byte aligned
  */
 int tk_swiglu_per_token_cast(const void *x, int x_dtype, int64_t R, int64_t H, void *out, void *sf, int64_t sf_ld,

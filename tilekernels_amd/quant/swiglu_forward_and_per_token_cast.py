@@ -66,7 +66,9 @@ def swiglu_forward_and_per_token_cast(
     out_sf = alloc_scaling_factors((num_expanded_tokens, hidden), out_config, dev)
     if num_expanded_tokens > 0:
         with torch.cuda.device(dev):
-            max_blocks = get_num_sms() * 4 if clamped_count is not None else 0
+            # the counting variant: at most 8 workgroups per compute unit, which then loop over tiles (every workgroup that
+            # clamped anything sends one atomic request to the counters, and those are served one at a time)
+            max_blocks = get_num_sms() * 8 if clamped_count is not None else 0
             rc = lib.tk_swiglu_per_token_cast(
                 x.data_ptr(), _ffi.dtype_code(x), num_expanded_tokens, hidden, out.data_ptr(), out_sf.data_ptr(),
                 sf_leading_dim(out_sf), num_per_channels, out_config.layout_code, int(round_sf),
