@@ -136,6 +136,7 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
             int use_clamp = p.use_clamp;
             asm volatile("" : "+s"(clamp_arg), "+s"(use_clamp));
             const float cl = use_clamp ? clamp_arg : __builtin_inff();
+            const float lo = cl >= 0.0f ? -cl : cl;      // (a negative limit makes every element the limit, as the two-step form does)
 #pragma unroll
             for (int r = 0; r < kPcRows; ++r) {
                 float g[8], u[8], a[8];
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     g[i] = __builtin_fminf(g[i], cl);
-                    u[i] = __builtin_fminf(__builtin_fmaxf(u[i], -cl), cl);
+                    u[i] = __builtin_amdgcn_fmed3f(u[i], lo, cl);      // min(max(u, -cl), cl) in one instruction
                     a[i] = silu_mul<bf16_t>(g[i], u[i]);
                 }
                 // the activation is rounded to bf16 before it is quantised, as in the reference
