@@ -110,11 +110,12 @@ def test_swiglu_fp32_input_tiles(H, with_mask, mode):
 @pytest.mark.parametrize('rnd', [False, True])
 @pytest.mark.parametrize('with_weights', [False, True])
 @pytest.mark.parametrize('layout', ['row', 'col', 'packed'])
-@pytest.mark.parametrize('R,H', [(6144, 2048), (3076, 4096), (8192, 2048), (1600, 8192)])
+@pytest.mark.parametrize('R,H', [(6144, 2048), (3076, 4096), (8192, 2048), (1600, 8192), (10912, 1536), (5456, 2560), (32768, 512), (4096, 3584)])
 def test_swiglu_launches_that_end_in_smaller_waves(R, H, layout, with_weights, rnd, clamp):
-    """Unmasked bf16 batches of about one to three times the GPU's wave slots, H a multiple of 2048: the last rows are
+    """Unmasked bf16 batches of about one to three times the GPU's wave slots, H a multiple of 512: the last rows are
     handled by waves of two pieces and of one piece (a different kernel path with its own argument handling; with the
-    column-major layouts the four waves of a workgroup take four rows of the same pieces and store their scales together).
+    column-major layouts the four waves of a workgroup take four rows of the same pieces and store their scales together;
+    where H is no multiple of 2048 a wave's two pieces lie one below the other).
     Rows, weights, clamp and the power-of-two scales must come out as from the one-row waves."""
     if layout == 'packed' and not rnd:
         pytest.skip('packed scales are powers of two')

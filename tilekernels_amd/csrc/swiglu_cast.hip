@@ -170,29 +170,34 @@ __device__ __forceinline__ float row_weight(const SwigluParams &p, int row) {
     return (pos >= 0 && pos < p.num_weights) ? uniform_load(p.topk_weights + pos) : 0.0f;
 }
 
-// One wave on NP consecutive pieces of one row (no mask; CLAMP 0 or 1): what a wave of a T_ROW or T_ROWC tile does, for the
-// finer-grained waves at the end of a launch (see the tiled kernel).  Row-major scales are stored by the wave itself; with
-// ROWC (column-major layouts) the caller's four waves hold rows row0 - wave .. row0 - wave + 3 of the same pieces.
-template <typename InT, int CLAMP, int NP, bool WEIGHTED, bool ROWC = false>
+// One wave on NP pieces (no mask; CLAMP 0 or 1), for the finer-grained waves at the end of a launch (see the tiled kernel):
+// consecutive pieces of one row, as in a T_ROW or T_ROWC tile, or with STACK the same piece of NP consecutive rows, as in a
+// T_STACKED tile.  SF says where the scales go: 0 row-major, stored by the wave itself; 1 column-major layouts: the
+// workgroup's four waves hold consecutive rows of the same pieces (rows row0 - wave * (STACK ? NP : 1) onwards), their
+// scales meet in LDS and leave as runs along the rows; 2 whichever the layout argument says (read behind the loads).
+template <typename InT, int CLAMP, int NP, bool WEIGHTED, int SF = 0, bool STACK = false>
 __device__ __forceinline__ void swiglu_row_wave(SwigluParams p, int row0, int strip) {
     static_assert(CLAMP != 2, "the counting variant loops over tiles");
     static_assert(Raw8<InT>::kXchgBytes == 0, "inputs whose pieces need no exchange between lanes");
     constexpr int GPS = kStripCols / 128;
+    constexpr int SROWS = kWaves * (STACK ? NP : 1), SCOLS = STACK ? GPS : NP * GPS;      // staged scales of the workgroup
     using RS = RowScales<448, NP, 16>;
     const int lane = threadIdx.x & 63, own = lane & 15;
     const int col = strip * kStripCols + lane * 8;
+    const int64_t rstep = STACK ? 2 * (int64_t)p.H : 0;       // from piece to piece, in elements of the input
+    constexpr int cstep = STACK ? 0 : kStripCols;
     const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * (2 * (int64_t)p.H) + col;
-    // column-major layouts: the workgroup's four waves hold four consecutive rows of the same pieces; their scales meet in
-    // LDS and leave as runs along the rows
-    __shared__ uint32_t stage[ROWC ? kWaves : 1][ROWC ? NP * GPS : 1];
+    __shared__ uint32_t stage[SF ? SROWS : 1][SF ? SCOLS : 1];
     Raw8<InT> rg[NP], ru[NP];
 #pragma unroll
     for (int r = 0; r < NP; ++r) {
-        rg[r].load(x + r * kStripCols);
-        ru[r].load(x + r * kStripCols + p.H);
+        rg[r].load(x + r * rstep + r * cstep);
+        ru[r].load(x + r * rstep + r * cstep + p.H);
     }
-    fetch_late_arguments(p, CLAMP != 0, WEIGHTED, ROWC);
-    const float w = WEIGHTED ? row_weight(p, row0) : 0.0f;
+    fetch_late_arguments(p, CLAMP != 0, WEIGHTED, SF != 0);
+    float w[NP];
+#pragma unroll
+    for (int r = 0; r < NP; ++r) w[r] = WEIGHTED ? ((STACK || r == 0) ? row_weight(p, row0 + (STACK ? r : 0)) : w[0]) : 0.0f;
     ClampCounter<CLAMP> clamp;
     float v[NP][8], amax[NP];
 #pragma unroll
@@ -205,27 +210,34 @@ __device__ __forceinline__ void swiglu_row_wave(SwigluParams p, int row0, int st
         for (int i = 0; i < 8; ++i) v[r][i] = silu_mul<InT>(g[i], u[i]);
         if (WEIGHTED) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[r][i] = v[r][i] * w;
+            for (int i = 0; i < 8; ++i) v[r][i] = v[r][i] * w[r];
         }
         amax[r] = group_allmax<16>(absmax8(v[r]));
     }
     RS rs;
     rs.compute(amax, p.floor_, p.round_sf != 0, lane);
-    // lane j (< A) of a group computed the scale of piece c*A + j; the wave's scales form one run of NP * 4 floats
+    const bool staged = SF == 1 || (SF == 2 && p.sf.layout != TK_SF_ROW_F32);      // uniform over the launch
+    // lane j (< A) of a group computed the scale of piece c*A + j
     if (own < RS::A) {
 #pragma unroll
         for (int c = 0; c < RS::NC; ++c) {
-            if constexpr (ROWC)
-                stage[wave_id()][(c * RS::A + own) * GPS + (lane >> 4)] = p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
-            else
-                st_stream4(reinterpret_cast<float *>(p.sf.base) + (int64_t)row0 * p.sf.ld + (strip + c * RS::A + own) * GPS + (lane >> 4), f2u(rs.own[c].sf));
+            const int pc = c * RS::A + own;
+            if (SF != 0 && staged) {
+                if (STACK) stage[wave_id() * NP + pc][lane >> 4] = p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
+                else stage[wave_id()][pc * GPS + (lane >> 4)] = p.sf.layout == TK_SF_COL_UE8M0 ? rs.own[c].e8 : f2u(rs.own[c].sf);
+            } else {
+                st_stream4(reinterpret_cast<float *>(p.sf.base) + (int64_t)(row0 + (STACK ? pc : 0)) * p.sf.ld + (strip + (STACK ? 0 : pc)) * GPS + (lane >> 4),
+                           f2u(rs.own[c].sf));
+            }
         }
     }
 #pragma unroll
-    for (int r = 0; r < NP; ++r) quantise_store8<TK_E4M3, false>(v[r], rs.inv[r], p.out + (int64_t)row0 * p.H, col + r * kStripCols);
-    if constexpr (ROWC) {
-        __syncthreads();
-        sf_store_tile_colmajor<kWaves, NP * GPS>(p.sf, stage, row0 - wave_id(), strip * GPS);
+    for (int r = 0; r < NP; ++r) quantise_store8<TK_E4M3, false>(v[r], rs.inv[r], p.out + (int64_t)(row0 + (STACK ? r : 0)) * p.H, col + r * cstep);
+    if constexpr (SF != 0) {
+        if (staged) {
+            __syncthreads();
+            sf_store_tile_colmajor<SROWS, SCOLS>(p.sf, stage, row0 - wave_id() * (STACK ? NP : 1), strip * GPS);
+        }
     }
 }
 
@@ -244,7 +256,7 @@ __device__ __forceinline__ void swiglu_row_wave(SwigluParams p, int row0, int st
 enum { T_STACKED = 0, T_ROW = 2, T_ROWC = 3 };
 
 // ONECOL: the grid is known to be a single column of tiles (else it is found out at run time)
-// TAILED (T_ROW and T_ROWC tiles of four-piece waves, exact grids): the launch ends in finer-grained waves.  The grid's row tiles
+// TAILED (tiles of four-piece waves, exact grids): the launch ends in finer-grained waves.  The grid's row tiles
 // come in three runs: `yb` workgroups of one-row waves as described above, then `ym` workgroups whose waves take two
 // pieces, then workgroups whose waves take one; all cover the rows in order.  The requests of a launch are served
 // roughly in the order they were made, so what arrives last belongs to the last workgroups; with whole rows per wave
@@ -258,12 +270,16 @@ enum { T_STACKED = 0, T_ROW = 2, T_ROWC = 3 };
 // the mask pointer (these launches have no mask) carries the leading dimension of the scales.  TAILED: 1 without, 2 with
 // routing weights.  T_ROWC tiles end the same way, with the four waves of a workgroup on four consecutive rows of the same
 // two pieces or one piece (swiglu_row_wave<..., ROWC>), so that their scales still leave as runs along the rows; layout
-// and group count of the scales are among the arguments read behind the loads.  bf16, us per call without / with,
+// and group count of the scales are among the arguments read behind the loads.  T_STACKED tiles (H a multiple of 512 but
+// not of 2048) end in workgroups of 4 x 2 rows and then 4 x 1 rows of one 512-column strip, a wave's two pieces one below
+// the other as in the tile (row-major scales, without / with: [10912, 2 x 1536] 14.57 / 14.31, [6544, 2 x 2560] 14.71 / 14.29,
+// [16384, 2 x 1536] 20.89 / 20.34, [2048, 2 x 7168] 13.52 / 12.97, [49152, 2 x 512] 20.96 / 20.35; packed: 14.46 / 14.31,
+// 14.42 / 14.20, 20.78 / 20.39, 13.12 / 12.83, 20.95 / 20.47).  bf16, us per call without / with,
 // column-major fp32 scales: [8192, 2 x 2048] 15.39 / 14.74, [4096, 2 x 4096] 15.34 / 14.86, [12288, 2 x 2048] 21.40 / 20.89,
 // [16384, 2 x 2048] 27.53 / 27.13; packed UE8M0: 14.79 / 14.36, 14.70 / 14.47, 21.11 / 20.61, 27.18 / 26.88.
 template <typename InT, int CLAMP, int RPW, int TILE, bool FULL_GRID, bool MASK, bool ONECOL, int TAILED = 0>
 __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void swiglu_cast_kernel(TK_SWIGLU_KERNEL_ARGS) {
-    static_assert(!TAILED || ((TILE == T_ROW || TILE == T_ROWC) && FULL_GRID && !MASK && CLAMP != 2 && RPW == 4), "tail waves: exact unmasked grids of one-row waves of four pieces");
+    static_assert(!TAILED || (FULL_GRID && !MASK && CLAMP != 2 && RPW == 4), "tail waves: exact unmasked grids of four-piece waves");
     if constexpr (TAILED) {
         // a_nwaves: waves per workgroup (bits 0-3), column tiles (4-15), two-piece workgroups (16-31); a_tiles_k: one-row workgroups
         const int yb = a_tiles_k, ym = (int)((unsigned)a_nwaves >> 16);
@@ -276,18 +292,29 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
             const int strip0 = tile_grid_col(one_col) * RPW, wave = wave_id();
             const int rb = yb * p.nwaves;                       // rows done by one-row waves
             int row, strip;
-            if constexpr (TILE == T_ROWC) {
+            if constexpr (TILE == T_STACKED) {
+                // stacked tiles: a wave's pieces lie one below the other; workgroups of 4 x 2 rows, then of 4 x 1 row, of one strip
+                strip = tile_grid_col(one_col);
+                const int rbs = yb * (kWaves * RPW);
+                if (y - yb < ym) {
+                    row = rbs + (y - yb) * (2 * kWaves) + wave * 2;
+                    swiglu_row_wave<InT, CLAMP, 2, TAILED == 2, 2, true>(p, row, strip);
+                } else {
+                    row = rbs + ym * (2 * kWaves) + (y - yb - ym) * kWaves + wave;
+                    if (row < p.R) swiglu_row_wave<InT, CLAMP, 1, TAILED == 2, 2, true>(p, row, strip);    // (whole workgroups overhang)
+                }
+            } else if constexpr (TILE == T_ROWC) {
                 // four rows per workgroup, one per wave, the same pieces in each
                 if (y - yb < ym) {
                     const int sub = y - yb;                         // two workgroups per four rows
                     row = rb + (sub >> 1) * kWaves + wave;
                     strip = strip0 + (sub & 1) * 2;
-                    swiglu_row_wave<InT, CLAMP, 2, TAILED == 2, true>(p, row, strip);
+                    swiglu_row_wave<InT, CLAMP, 2, TAILED == 2, 1>(p, row, strip);
                 } else {
                     const int sub = y - yb - ym;                    // four workgroups per four rows
                     row = rb + ym * 2 + (sub >> 2) * kWaves + wave;
                     strip = strip0 + (sub & 3);
-                    if (row < p.R) swiglu_row_wave<InT, CLAMP, 1, TAILED == 2, true>(p, row, strip);    // (whole workgroups overhang)
+                    if (row < p.R) swiglu_row_wave<InT, CLAMP, 1, TAILED == 2, 1>(p, row, strip);    // (whole workgroups overhang)
                 }
             } else if (y - yb < ym) {
                 const int sub = (y - yb) * p.nwaves + wave;     // two waves per row
@@ -395,7 +422,7 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
         }
 
         // (in this variant the fetch of the later arguments starts at the head of the kernel, where its paths part)
-        if constexpr (TAILED != 0) fetch_late_arguments(p, CLAMP != 0, TAILED == 2, TILE == T_ROWC);
+        if constexpr (TAILED != 0) fetch_late_arguments(p, CLAMP != 0, TAILED == 2, TILE != T_ROW);
         if constexpr (FULL && XB != 0) {
 #pragma unroll
             for (int r = 0; r < RPW; ++r) {
@@ -682,7 +709,7 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
     // run-time test costs the [8192, 2 x 2048] call 0.2 us
     constexpr bool ROWWISE = TILE == T_ROW || TILE == T_ROWC;
     const bool onecol = ROWWISE && p.tiles_k == 1;
-    if constexpr ((TILE == T_ROW || TILE == T_ROWC) && CLAMP != 2 && RPW == 4) {
+    if constexpr (CLAMP != 2 && RPW == 4) {
         // Finer-grained waves at the end of the launch (see the kernel): the last rows by two-piece waves, 2.2 times the GPU's
         // wave slots of them but at most 55 % of the rows, and of those the last by one-piece waves, 0.6 times the slots, at
         // most 15 % of the rows.  For launches of 0.75 to 3.5 times the GPU's wave slots in one-row waves, where it was
@@ -691,10 +718,17 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
         // 14.77 / 14.32, [24576, 2 x 2048] 42.92 / 42.54; smaller and larger launches lose with it ([4096, 2 x 2048] 8.11 / 8.48,
         // [32768, 2 x 2048] 57.37 / 57.71), and so does a masked batch ([48128, 2 x 2048], a third of the rows padding, 59.9 / 61.8).
         const int64_t slots = wave_slots(), ppr = p.H / kStripCols, row_waves = (int64_t)p.R * ppr / RPW;
-        const int rs = (int)std::min<int64_t>((int64_t)p.R * 15 / 100, slots * 6 / 10 / ppr) / 4 * 4;
-        const int rm = (int)std::min<int64_t>((int64_t)p.R * 55 / 100, slots * 22 / 10 / ppr) / 4 * 4;
-        const int rb = p.R - rm - rs;
-        const int64_t ym = (int64_t)rm * 2 / waves, ys = (int64_t)rs * 4 / waves, yb = rb / waves;
+        int rs = (int)std::min<int64_t>((int64_t)p.R * 15 / 100, slots * 6 / 10 / ppr) / 4 * 4;
+        int rm = (int)std::min<int64_t>((int64_t)p.R * 55 / 100, slots * 22 / 10 / ppr) / 4 * 4;
+        int rb = p.R - rm - rs;
+        int64_t ym = (int64_t)rm * 2 / waves, ys = (int64_t)rs * 4 / waves, yb = rb / waves;
+        if constexpr (TILE == T_STACKED) {
+            // stacked tiles of 16 rows, then workgroups of 8 rows (two per wave), then of 4 rows, each on one strip of 512 columns
+            rs = rs / 8 * 8;
+            rb = (p.R - rm - rs) / rows * rows;
+            rm = p.R - rb - rs;
+            yb = rb / rows; ym = rm / (2 * kWaves); ys = rs / kWaves;
+        }
         if (full && !p.pos_to_expert && row_waves * 4 >= slots * 3 && row_waves * 2 <= slots * 7 && rs > 0 && p.tiles_k <= 0xFFF &&
             ym <= 0xFFFF) {
             const dim3 tgrid = tile_grid(p.tiles_k, (int)(yb + ym + ys));
