@@ -355,9 +355,10 @@ def op_swiglu_weighted():
     return launch, algo, nbytes(x, out, sf), cpu
 
 
-def op_swiglu_dense(R, H, packed_col_major):
+def op_swiglu_dense(R, H, packed_col_major, count_clamp=False):
     """The headline operator on dense rows of other shapes and scale layouts: packed UE8M0 column-major scales (the layout a
-    block-scaled GEMM consumes) at the headline shape, and short rows (H = 768)."""
+    block-scaled GEMM consumes) at the headline shape, short rows (H = 768), rows of three 512-column pieces (H = 1536), and
+    with a clamp at 6 whose hits are counted (clamped_count; N(0,1) data, so next to nothing is clamped)."""
     def build():
         import tilekernels_amd as tk
         from tilekernels_amd import _ffi
@@ -368,18 +369,23 @@ def op_swiglu_dense(R, H, packed_col_major):
         oc = get_cast_output_config('e4m3', (1, 128), packed_col_major, packed_col_major, packed_col_major)
         sf = alloc_scaling_factors((R, H), oc, x.device)
         stream = _ffi.current_stream(x.device)
+        counts = torch.zeros(3, dtype=torch.int64, device='cuda')
+        cap = 8 * torch.cuda.get_device_properties(x.device).multi_processor_count      # what the Python wrapper passes
 
         def launch():
             rc = lib.tk_swiglu_per_token_cast(x.data_ptr(), _ffi.TK_BF16, R, H, out.data_ptr(), sf.data_ptr(), sf_leading_dim(sf), 128,
-                                              oc.layout_code, int(packed_col_major), -1.0, 0, 0, 0, 0, 0, 0.0, 0, 0, stream)
+                                              oc.layout_code, int(packed_col_major), -1.0, 0, 0, 0, 0, int(count_clamp), 6.0 if count_clamp else 0.0,
+                                              counts.data_ptr() if count_clamp else 0, cap if count_clamp else 0, stream)
             assert rc == 0, rc
         b = nbytes(x, out) + R * (H // 128) * (1 if packed_col_major else 4)
 
         def cpu():
             from oracle import torch_ref
             xc = x.cpu()
+            cc = torch.zeros(3, dtype=torch.int64) if count_clamp else None
             return lambda: torch_ref.swiglu_forward_and_per_token_cast(xc, 'e4m3', 128, use_tma_aligned_col_major_sf=packed_col_major,
-                                                                       round_sf=packed_col_major, use_packed_ue8m0=packed_col_major)
+                                                                       round_sf=packed_col_major, use_packed_ue8m0=packed_col_major,
+                                                                       swiglu_clamp_value=6.0 if count_clamp else None, clamped_count=cc)
         return launch, b, b, cpu
     return build
 
@@ -493,6 +499,10 @@ OPS = [
        'swiglu_forward_and_per_token_cast e4m3 1x128, MoE-expanded bf16 [R,4096] with mask and routing weights', op_swiglu_weighted),
     Op('swiglu_forward_and_per_token_cast_packed_sf', 'swiglu_forward_and_per_token_cast e4m3 1x128, packed UE8M0 column-major scales, bf16 [8192,4096]',
        op_swiglu_dense(8192, 2048, True)),
+    Op('swiglu_forward_and_per_token_cast_clamped_count', 'swiglu_forward_and_per_token_cast e4m3 1x128 with a clamp and clamped_count, bf16 [8192,4096]',
+       op_swiglu_dense(8192, 2048, False, True)),
+    Op('swiglu_forward_and_per_token_cast_h1536', 'swiglu_forward_and_per_token_cast e4m3 1x128, rows of three pieces: bf16 [10912,3072]',
+       op_swiglu_dense(10912, 1536, False)),
     Op('swiglu_forward_and_per_token_cast_h768', 'swiglu_forward_and_per_token_cast e4m3 1x128, short rows: bf16 [32768,1536]',
        op_swiglu_dense(32768, 768, False), floor=(32768 * 1536 * 2, 16, 4, 4)),
     Op('expand_to_fused_with_sf', 'expand_to_fused_with_sf e4m3 [4096,4096] + 1x128 scales -> [R,4096], top-8 of 256 experts, pad 128',
