@@ -187,3 +187,18 @@ def test_swiglu_empty():
     assert c.shape == (0, 256) and s.shape == (0, 2)
     c, s = tk.quant.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, use_tma_aligned_col_major_sf=True, round_sf=True, use_packed_ue8m0=True)
     assert c.shape == (0, 256) and s.shape == (0, 1) and s.dtype == torch.int32
+
+
+@pytest.mark.parametrize('gate', [0.5, 3.0, -1.0])
+def test_swiglu_rows_that_share_one_gate_value(gate):
+    """Every element of a group is the same factor silu(gate) times its up value, so 448 * v / amax falls on exact rounding
+    boundaries of E4M3 for many elements, and the last bit of the factor decides which way they go: the quotient
+    gate / (1 + exp(-gate)) has to be the correctly rounded one (an uncorrected reciprocal-multiply puts 1e-3 of the codes on
+    the other side for gates 0.5 and 3.0, ten times the budget)."""
+    tk = _tk()
+    R, H = 2048, 2048
+    g = torch.Generator().manual_seed(5)
+    x = torch.cat([torch.full((R, H), gate), torch.randn((R, H), generator=g)], 1).to(torch.bfloat16)
+    want = torch_ref.swiglu_forward_and_per_token_cast(x, 'e4m3', 128)
+    got = tk.quant.swiglu_forward_and_per_token_cast(x.cuda(), 'e4m3', 128)
+    check_fused(got, want, H // 128, False, f'gate {gate} everywhere')
