@@ -186,13 +186,20 @@ __device__ __forceinline__ void swiglu_row_wave(SwigluParams p, int row0, int st
     const int col = strip * kStripCols + lane * 8;
     const int64_t rstep = STACK ? 2 * (int64_t)p.H : 0;       // from piece to piece, in elements of the input
     constexpr int cstep = STACK ? 0 : kStripCols;
-    const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * (2 * (int64_t)p.H) + col;
+    // (row, column and H are non-negative 32-bit numbers: unsigned, the row offset is one 32 x 32 -> 64-bit product and nothing
+    // needs a sign extension on the way to the loads)
+    // The addresses are a wave-uniform 64-bit base (in scalar registers) plus a 32-bit byte offset per lane, which is the form
+    // the load instruction takes as it is; a 64-bit address per lane costs two more vector instructions before every load.
+    const uint32_t uh = (uint32_t)p.H;
+    const uint8_t *xrow = reinterpret_cast<const uint8_t *>(p.x) + (uint64_t)(uint32_t)row0 * (2u * uh * (uint32_t)sizeof(InT));
+    const uint32_t lane_off = (uint32_t)strip * (uint32_t)(kStripCols * sizeof(InT)) + (uint32_t)lane * (uint32_t)(8 * sizeof(InT));
     __shared__ uint32_t stage[SF ? SROWS : 1][SF ? SCOLS : 1];
     Raw8<InT> rg[NP], ru[NP];
 #pragma unroll
     for (int r = 0; r < NP; ++r) {
-        rg[r].load(x + r * rstep + r * cstep);
-        ru[r].load(x + r * rstep + r * cstep + p.H);
+        const uint8_t *xg = xrow + (uint64_t)r * (uint64_t)rstep * sizeof(InT) + (uint32_t)(r * cstep) * (uint32_t)sizeof(InT);
+        rg[r].load(xg + lane_off);
+        ru[r].load(xg + uh * (uint32_t)sizeof(InT) + lane_off);
     }
     fetch_late_arguments(p, CLAMP != 0, WEIGHTED, SF != 0);
     float w[NP];
@@ -290,7 +297,7 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
         if (y >= yb) {
             TK_SWIGLU_KERNEL_UNPACK_EARLY;
             const int strip0 = tile_grid_col(one_col) * RPW, wave = wave_id();
-            const int rb = yb * p.nwaves;                       // rows done by one-row waves
+            const int rb = yb * kWaves;                         // rows done by one-row waves (these launches run four waves per workgroup)
             int row, strip;
             if constexpr (TILE == T_STACKED) {
                 // stacked tiles: a wave's pieces lie one below the other; workgroups of 4 x 2 rows, then of 4 x 1 row, of one strip
@@ -317,13 +324,13 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
                     if (row < p.R) swiglu_row_wave<InT, CLAMP, 1, TAILED == 2, 1>(p, row, strip);    // (whole workgroups overhang)
                 }
             } else if (y - yb < ym) {
-                const int sub = (y - yb) * p.nwaves + wave;     // two waves per row
+                const int sub = (y - yb) * kWaves + wave;       // two waves per row
                 row = rb + (sub >> 1);
                 strip = strip0 + (sub & 1) * 2;
                 swiglu_row_wave<InT, CLAMP, 2, TAILED == 2>(p, row, strip);
             } else {
-                const int sub = (y - yb - ym) * p.nwaves + wave;      // four waves per row
-                row = rb + ((ym * p.nwaves) >> 1) + (sub >> 2);
+                const int sub = (y - yb - ym) * kWaves + wave;        // four waves per row
+                row = rb + ((ym * kWaves) >> 1) + (sub >> 2);
                 strip = strip0 + (sub & 3);
                 if (row < p.R) swiglu_row_wave<InT, CLAMP, 1, TAILED == 2>(p, row, strip);    // (the grid may overhang along z)
             }
@@ -347,7 +354,7 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
     // counters); every other variant has one workgroup per tile on a 2-D grid, which keeps integer
     // divisions and further kernel-argument loads out of the path to the first memory load.
     constexpr bool LOOP = CLAMP == 2;
-    const int nwaves = DIRECT ? p.nwaves : kWaves;
+    const int nwaves = (DIRECT && !TAILED) ? p.nwaves : kWaves;      // (launches that end in smaller waves run four waves per workgroup)
     const int rows = DIRECT ? nwaves : ROWS;
     using RS = RowScales<448, RPW, 16>;
     __shared__ uint32_t stage[DIRECT ? 1 : ROWS][DIRECT ? 1 : SGPR];
@@ -372,7 +379,8 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
         if constexpr (ROWGUARD) {
             if (row0 >= p.R) return;
         }
-        const InT *x = reinterpret_cast<const InT *>(p.x) + (int64_t)row0 * (2 * (int64_t)p.H) + col;
+        const uint32_t uh = (uint32_t)p.H;      // (unsigned: see swiglu_row_wave)
+        const InT *x = reinterpret_cast<const InT *>(p.x) + (uint64_t)(uint32_t)row0 * (2u * uh) + (uint32_t)col;
         constexpr int kRowStep = ROW ? 0 : 1, kColStep = ROW ? kStripCols : 0;
 
         Raw8<InT> rg[RPW], ru[RPW];
@@ -397,17 +405,21 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
             live[r] = (FULL || row0 + r * kRowStep < p.R) && expert[r] >= 0;
-            const InT *xr = x + (int64_t)(r * kRowStep) * (2 * (int64_t)p.H) + r * kColStep;
+            const InT *xr = x + (uint64_t)(uint32_t)(r * kRowStep) * (2u * uh) + r * kColStep;
             const bool piece_ok = FULL || col + r * kColStep < p.H;
             if (FULL && !MASK) {
-                rg[r].template load_run<64>(xr, lane);
-                ru[r].template load_run<64>(xr + p.H, lane);
+                // (a wave-uniform 64-bit base plus a 32-bit byte offset per lane: see swiglu_row_wave)
+                const uint8_t *xg = reinterpret_cast<const uint8_t *>(p.x) + (uint64_t)(uint32_t)(row0 + r * kRowStep) * (2u * uh * (uint32_t)sizeof(InT)) +
+                                    (uint32_t)(r * kColStep) * (uint32_t)sizeof(InT);
+                const uint32_t lane_off = (uint32_t)strip * (uint32_t)(kStripCols * sizeof(InT)) + (uint32_t)lane * (uint32_t)(8 * sizeof(InT));
+                rg[r].template load_run<64>(xg + lane_off, lane);
+                ru[r].template load_run<64>(xg + uh * (uint32_t)sizeof(InT) + lane_off, lane);
             } else if (FULL && XB != 0) {
                 // (a padding row reads the first 2 KB of the matrix, as one run)
                 const bool ok = live[r];
                 const InT *src = ok ? xr : reinterpret_cast<const InT *>(p.x) + lane * 8;
                 rg[r].template load_run<64>(src, lane);
-                ru[r].template load_run<64>(ok ? xr + p.H : src, lane);
+                ru[r].template load_run<64>(ok ? xr + uh : src, lane);
                 if (!ok) { rg[r].zero(); ru[r].zero(); }
             } else {
                 // no branch around the loads (a branch would make the compiler wait for all eight loads
@@ -416,7 +428,7 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
                 const bool ok = live[r] && piece_ok;
                 const InT *src = ok ? xr : reinterpret_cast<const InT *>(p.x);
                 rg[r].load(src);
-                ru[r].load(ok ? xr + p.H : src);
+                ru[r].load(ok ? xr + uh : src);
                 if (!ok) { rg[r].zero(); ru[r].zero(); }
             }
         }
@@ -729,7 +741,7 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
             rm = p.R - rb - rs;
             yb = rb / rows; ym = rm / (2 * kWaves); ys = rs / kWaves;
         }
-        if (full && !p.pos_to_expert && row_waves * 4 >= slots * 3 && row_waves * 2 <= slots * 7 && rs > 0 && p.tiles_k <= 0xFFF &&
+        if (full && !p.pos_to_expert && waves == kWaves && row_waves * 4 >= slots * 3 && row_waves * 2 <= slots * 7 && rs > 0 && p.tiles_k <= 0xFFF &&
             ym <= 0xFFFF) {
             const dim3 tgrid = tile_grid(p.tiles_k, (int)(yb + ym + ys));
             p.nwaves = waves | (p.tiles_k << 4) | ((int)ym << 16);
