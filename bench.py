@@ -215,9 +215,52 @@ def time_gpu_graph(w: 'Workload', steps: int, warmup: int, chunk: int = 100):
     return wall, us, us, [a.elapsed_time(b) * 1e3 for a, b in ev]
 
 
-def time_gpu(w: 'Workload', steps: int, warmup: int):
+class RawEvents:
+    """HIP events made by the runtime itself (the copy of it that torch has loaded) with hipEventDisableSystemFence: such an
+    event is a time stamp in the stream and nothing else.  An ordinary event (torch's) also makes the kernels before it
+    visible to the host, and the kernel behind it starts about 2 us later for that: a tenth of a microsecond per launch
+    in a region of 20 launches with one event behind the first, nothing to speak of in a region of thousands."""
+    NO_SYSTEM_FENCE = 0x20000000
+
+    def __init__(self):
+        import ctypes
+        self.ct = ctypes
+        hip = ctypes.CDLL(os.path.join(os.path.dirname(torch.__file__), 'lib', 'libamdhip64.so'))
+        hip.hipEventCreateWithFlags.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint]
+        hip.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        hip.hipEventQuery.argtypes = [ctypes.c_void_p]
+        hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+        hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip = hip
+
+    def make(self):
+        e = self.ct.c_void_p()
+        if self.hip.hipEventCreateWithFlags(self.ct.byref(e), self.NO_SYSTEM_FENCE) != 0:
+            raise RuntimeError('hipEventCreateWithFlags failed')
+        return e
+
+    def record(self, e, stream: int) -> None:
+        if self.hip.hipEventRecord(e, self.ct.c_void_p(stream)) != 0:
+            raise RuntimeError('hipEventRecord failed')
+
+    def done(self, e) -> bool:
+        return self.hip.hipEventQuery(e) == 0
+
+    def elapsed_us(self, a, b) -> float:
+        ms = self.ct.c_float()
+        if self.hip.hipEventElapsedTime(self.ct.byref(ms), a, b) != 0:
+            raise RuntimeError('hipEventElapsedTime failed')
+        return ms.value * 1e3
+
+    def destroy(self, *events) -> None:
+        for e in events:
+            self.hip.hipEventDestroy(e)
+
+
+def time_gpu(w: 'Workload', steps: int, warmup: int, fenceless: bool = False):
     """Returns (wall seconds for `steps` launches, HIP-event microseconds per launch, the same with the first launch
-    left in, list of single-launch durations from per-launch event pairs).
+    left in, list of single-launch durations from per-launch event pairs).  `fenceless`: the three events of the
+    timed region are RawEvents instead of torch's.
 
     The timed region starts on an idle GPU (it follows a synchronisation), and the first launch needs a few
     microseconds to get there that are no part of any kernel's duration (a kernel trace does not show them either).
@@ -227,22 +270,32 @@ def time_gpu(w: 'Workload', steps: int, warmup: int):
     for i in range(warmup):
         w.launch(i)
     torch.cuda.synchronize()
-    e0, ef, e1 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
     todo = [w.calls[i % w.nsets] for i in range(steps)]
-    e0.record()          # torch's current stream is the stream the launches go to
+    if fenceless:
+        raw = RawEvents()
+        e0, ef, e1 = raw.make(), raw.make(), raw.make()
+        record, done = (lambda e: raw.record(e, w.main_stream)), raw.done
+        elapsed_us = raw.elapsed_us
+    else:
+        e0, ef, e1 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+        record, done = (lambda e: e.record()), (lambda e: e.query())      # torch's current stream is the stream the launches go to
+        elapsed_us = lambda a, b: a.elapsed_time(b) * 1e3
+    record(e0)
     t0 = time.perf_counter()
     for n, (fn, call_args) in enumerate(todo):
         if fn(*call_args) != 0:
             raise RuntimeError('launch failed')
         if n == 0:
-            ef.record()
-    e1.record()
-    while not e1.query():     # the end of the region is seen by polling: a blocking wait wakes up tens of microseconds late
+            record(ef)
+    record(e1)
+    while not done(e1):     # the end of the region is seen by polling: a blocking wait wakes up tens of microseconds late
         pass
     wall = time.perf_counter() - t0
     torch.cuda.synchronize()
-    region_all_us = e0.elapsed_time(e1) * 1e3 / steps
-    region_us = ef.elapsed_time(e1) * 1e3 / (steps - 1) if steps >= 4 else region_all_us
+    region_all_us = elapsed_us(e0, e1) / steps
+    region_us = elapsed_us(ef, e1) / (steps - 1) if steps >= 4 else region_all_us
+    if fenceless:
+        raw.destroy(e0, ef, e1)
     # single launches: one event pair around each (adds the cost of the two event records)
     n = min(steps, 200)
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
@@ -614,10 +667,11 @@ def cpu_baseline(w: Workload, budget_s: float = 12.0, min_runs: int = 3):
 
 
 def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_streams: bool = True, preheat_ms: float = 40.0,
-                 cpu_budget_s: float = 12.0, with_reference: bool = True, traffic: dict = None, graph: bool = False):
+                 cpu_budget_s: float = 12.0, with_reference: bool = True, traffic: dict = None, graph: bool = False,
+                 fenceless: bool = False):
     w = Workload(cfg)
     heated = preheat(w, preheat_ms)
-    wall, kern_us, kern_all_us, per = time_gpu_graph(w, steps, warmup) if graph else time_gpu(w, steps, warmup)
+    wall, kern_us, kern_all_us, per = time_gpu_graph(w, steps, warmup) if graph else time_gpu(w, steps, warmup, fenceless)
     ms_per_step = wall / steps * 1e3
     value = w.bytes / (wall / steps) / 1e9
     achieved = w.bytes / (kern_us * 1e-6) / 1e9
@@ -637,7 +691,7 @@ def bench_config(cfg: int, steps: int, warmup: int, with_cpu: bool, with_two_str
                                         else 'earlier rocprofv3 counter runs of this script (profiles/)'),
                      'kernel_us': round(kern_us, 3),
                      'timing': ('HIP events around replays of a HIP graph of launches on the rotating buffers (about 100 per replay), per launch' if graph else
-                                f'HIP events: from behind the first of the {steps} timed launches to the end of the region / {steps - 1} '
+                                f'HIP events{" without a system fence" if fenceless else ""}: from behind the first of the {steps} timed launches to the end of the region / {steps - 1} '
                                 '(the region starts on an idle GPU; what the first launch takes to get there is no kernel time)'
                                 if steps >= 4 else f'HIP events around the {steps} timed launches / {steps}'),
                      'kernel_us_first_launch_included': round(kern_all_us, 3),
@@ -709,6 +763,9 @@ def main():
     ap.add_argument('--graph', action='store_true',
                     help='enqueue the timed launches of --config from a HIP graph (100 launches per replay) instead of from the host: '
                          'for runs under a profiler, where the host is slower than the kernel')
+    ap.add_argument('--fenceless-events', action='store_true',
+                    help='time the region of --config with HIP events created with hipEventDisableSystemFence (time stamps only) instead '
+                         'of torch\'s: the event behind the first launch then does not hold up the second; matters for regions of tens of launches')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run plain device copies of known size (reference kernel for hardware-counter runs)')
     args = ap.parse_args()
@@ -737,7 +794,7 @@ def main():
         sys.exit('bench.py needs a GPU')
     two = not args.single_stream_only
     line = bench_config(args.config, args.steps, args.warmup, not args.no_cpu, two, args.preheat_ms, 12.0, two, traffic.get(args.config),
-                        args.graph)
+                        args.graph, args.fenceless_events)
     if traffic:
         line['traffic_measurement'] = {str(c): t for c, t in traffic.items()}
     if not args.only:
