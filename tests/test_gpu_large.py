@@ -203,3 +203,38 @@ def test_more_row_tiles_than_one_grid_plane():
             part = tk.quant.swiglu_forward_and_per_token_cast(x[a:b].contiguous(), 'e4m3', 128, **kw)
             check_fused(part, want, H // 128, bool(kw), f'window [{a}:{b}] alone')
             assert torch.equal(dense_bytes(got[0][a:b].cpu()), dense_bytes(part[0].cpu())), f'codes[{a}:{b}] {kw}'
+
+
+@pytest.mark.parametrize('dtype,H', [(torch.bfloat16, 4096), (torch.float32, 2048)], ids=['bf16', 'fp32'])
+@pytest.mark.parametrize('clamp', [None, 0.75])
+def test_masked_swiglu_with_more_rows_than_one_grid_plane(dtype, H, clamp):
+    """A masked batch in row-wise tiles runs one row per workgroup: with two columns of tiles and more than 32768 rows the
+    grid gets a second, partly empty plane, whose surplus workgroups must leave without touching anything."""
+    tk = _tk()
+    R = 32768 + 1203
+    g = torch.Generator(device='cuda').manual_seed(13)
+    x = (torch.randn((R, 2 * H), generator=g, device='cuda') * 2).to(dtype)
+    pe = torch.zeros((R,), dtype=torch.int32, device='cuda')
+    pe[3::5] = -1
+    guard = 64
+    codes_buf = torch.full((R + guard, H), 0x5A, dtype=torch.uint8, device='cuda')
+    kw = dict(swiglu_clamp_value=clamp)
+    codes, sf = tk.quant.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, pos_to_expert=pe, **kw)
+    for a, b in [(0, 16), (32768 - 8, 32768 + 8), (R - 16, R)]:
+        xw, pw = x[a:b].cpu(), pe[a:b].cpu()
+        want = torch_ref.swiglu_forward_and_per_token_cast(xw, 'e4m3', 128, pos_to_expert=pw, **kw)
+        dead = pw < 0
+        assert torch.all(codes[a:b].cpu().view(torch.uint8)[dead] == 0) and torch.all(sf[a:b].cpu()[dead] == 0)
+        live = ~dead
+        check_fused((codes[a:b][live.cuda()], sf[a:b][live.cuda()].contiguous()),
+                    (want[0][live], want[1][live].contiguous()), H // 128, False, f'rows[{a}:{b}]')
+    # the same call through the C ABI into a buffer with guard rows behind it: nothing beyond row R is written
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    sf2 = torch.empty_like(sf)
+    rc = lib.tk_swiglu_per_token_cast(x.data_ptr(), _ffi.dtype_code(x), R, H, codes_buf.data_ptr(), sf2.data_ptr(), H // 128, 128, 0, 0, -1.0,
+                                      0, 0, 0, pe.data_ptr(), int(clamp is not None), float(clamp or 0.0), 0, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    assert torch.equal(codes_buf[:R], codes.view(torch.uint8)) and torch.equal(sf2, sf)
+    assert bool((codes_buf[R:] == 0x5A).all()), 'rows beyond the batch were written'

@@ -79,7 +79,7 @@ def test_stream_floor_rejects_bad_shapes():
     assert lib.tk_stream_floor(0, 0, 1024, 0, 0, 0, None) == 0          # no rows: nothing to do
 
 
-@pytest.mark.parametrize('rows,cols,two', [(37, 2048, True), (64, 4096, False), (9, 3072, True)])
+@pytest.mark.parametrize('rows,cols,two', [(37, 2048, True), (64, 4096, False), (9, 3072, True), (21, 1024, False)])
 def test_stream_floor_timeline_stamps_every_wave(rows, cols, two):
     """The time-stamped variant writes the same output and, per wave, four non-decreasing times and its place."""
     from tilekernels_amd import _ffi

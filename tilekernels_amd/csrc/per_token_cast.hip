@@ -332,25 +332,30 @@ static void launch_per_token_rowgroup(PerTokenParams &p, hipStream_t stream) {
         if (waves <= kWaves) { iters = it; threads = (int)waves * 64; break; }
     }
     p.geom = threads;
-#define TK_ROWGROUP_LAUNCH(I)                                                                                                             \
-    do {                                                                                                                                  \
-        if (threads == kThreads && p.K == (I) * kThreads * 8)                                                                             \
-            hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT, I, kThreads, (I) != 0>), dim3(p.M), dim3(threads), 0, stream, TK_PT_LAUNCH_ARGS(p)); \
-        else if (threads == kThreads)                                                                                                     \
-            hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT, I, kThreads, false>), dim3(p.M), dim3(threads), 0, stream, TK_PT_LAUNCH_ARGS(p)); \
-        else                                                                                                                              \
-            hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT, I, 0, false>), dim3(p.M), dim3(threads), 0, stream, TK_PT_LAUNCH_ARGS(p));   \
+    // PARTIAL: the thread count template argument of a row that needs fewer than four waves (0: read from the arguments).  With 4 and
+    // 8 pieces, and in two passes, a row always takes all four waves (the piece count before would have covered it otherwise).
+#define TK_ROWGROUP_LAUNCH_NT(I, NT, EXACT) \
+    hipLaunchKernelGGL((per_token_rowgroup_kernel<InT, FMT, I, NT, EXACT>), dim3(p.M), dim3(threads), 0, stream, TK_PT_LAUNCH_ARGS(p))
+#define TK_ROWGROUP_LAUNCH(I, PARTIAL)                                              \
+    do {                                                                            \
+        if (threads == kThreads && (I) != 0 && p.K == (I) * kThreads * 8)           \
+            TK_ROWGROUP_LAUNCH_NT(I, kThreads, (I) != 0);                           \
+        else if (threads == kThreads)                                               \
+            TK_ROWGROUP_LAUNCH_NT(I, kThreads, false);                              \
+        else                                                                        \
+            TK_ROWGROUP_LAUNCH_NT(I, PARTIAL, false);                               \
     } while (0)
     switch (iters) {
-        case 1: TK_ROWGROUP_LAUNCH(1); break;
-        case 2: TK_ROWGROUP_LAUNCH(2); break;
-        case 3: TK_ROWGROUP_LAUNCH(3); break;
-        case 4: TK_ROWGROUP_LAUNCH(4); break;
-        case 6: TK_ROWGROUP_LAUNCH(6); break;
-        case 8: TK_ROWGROUP_LAUNCH(8); break;
-        default: TK_ROWGROUP_LAUNCH(0); break;
+        case 1: TK_ROWGROUP_LAUNCH(1, 0); break;
+        case 2: TK_ROWGROUP_LAUNCH(2, 0); break;
+        case 3: TK_ROWGROUP_LAUNCH(3, 0); break;
+        case 4: TK_ROWGROUP_LAUNCH(4, kThreads); break;
+        case 6: TK_ROWGROUP_LAUNCH(6, 0); break;
+        case 8: TK_ROWGROUP_LAUNCH(8, kThreads); break;
+        default: TK_ROWGROUP_LAUNCH(0, kThreads); break;
     }
 #undef TK_ROWGROUP_LAUNCH
+#undef TK_ROWGROUP_LAUNCH_NT
 }
 
 // Short rows (plain inputs): the strips of the tiled kernels are 512 columns wide, so a row of 576 columns keeps 72 of

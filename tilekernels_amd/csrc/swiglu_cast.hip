@@ -772,8 +772,13 @@ static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t str
                                TK_SWIGLU_LAUNCH_ARGS(p));                                                                       \
     } while (0)
     if (p.pos_to_expert) {
-        if (full) TK_SWIGLU_LAUNCH(true, true);
-        else TK_SWIGLU_LAUNCH(false, true);
+        // A masked batch in row-wise tiles takes one row per workgroup, so its grid fits unless it has more than one plane of
+        // row tiles (several columns of tiles, more than 32768 rows); the counting variant's grid is flat and always fits.
+        constexpr bool kAlwaysExact = TILE == T_ROW && CLAMP == 2;
+        if (full || kAlwaysExact) TK_SWIGLU_LAUNCH(true, true);
+        else if constexpr (TILE == T_ROW && !kAlwaysExact)
+            hipLaunchKernelGGL((swiglu_cast_kernel<InT, CLAMP, RPW, TILE, false, true, false>), grid, block, 0, stream, TK_SWIGLU_LAUNCH_ARGS(p));
+        else if constexpr (!kAlwaysExact) TK_SWIGLU_LAUNCH(false, true);
     } else {
         if (full) TK_SWIGLU_LAUNCH(true, false);
         else TK_SWIGLU_LAUNCH(false, false);
