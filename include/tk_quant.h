@@ -142,7 +142,8 @@ int tk_check_per_block_cast(const void *x, int x_dtype, int64_t M, int64_t K, co
  *                       anything sends one atomic request to the counters, and requests to one line are served
  *                       one at a time; the Python wrapper passes 8 per compute unit); <= 0 or without
  *                       clamped_count: one workgroup per tile
- *   requirements        H % 128 == 0; group == 128, or group == H with TK_SF_ROW_F32; x 16-byte aligned
+ *   requirements        H % 128 == 0; group == 128, or group == H with TK_SF_ROW_F32; x 16-byte aligned;
+ *                       a row of x (2 H elements) shorter than 4 GiB (TK_ERR_TOO_LARGE otherwise)
  */
 int tk_swiglu_per_token_cast(const void *x, int x_dtype, int64_t R, int64_t H, void *out, void *sf, int64_t sf_ld,
                              int group, int sf_layout, int round_sf, float sf_clamp_min,

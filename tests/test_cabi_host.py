@@ -127,6 +127,8 @@ def test_swiglu_validation(lib):
     assert check_sw(lib, group=256) == GROUP
     assert check_sw(lib, H=2000) == SHAPE
     assert check_sw(lib, R=-5) == SHAPE
+    assert check_sw(lib, dt=1, H=2 ** 29) == LARGE                      # an fp32 row of 4 GiB: byte offsets inside a row are 32-bit
+    assert check_sw(lib, dt=0, H=2 ** 29, sf_ld=2 ** 22) == OK
     assert check_sw(lib, cnt=P) == MODE                                 # counters need a clamp
     assert check_sw(lib, cnt=P, use_clamp=1, clamp=1.0) == OK
     assert check_sw(lib, cnt=P + 4, use_clamp=1, clamp=1.0) == ALIGN

@@ -861,6 +861,7 @@ extern "C" int tk_check_swiglu_per_token_cast(const void *x, int x_dtype, int64_
     if (sf_layout == TK_SF_COL_UE8M0 && !round_sf) return TK_ERR_BAD_LAYOUT;
     if (R < 0 || H <= 0 || H % 128 != 0) return TK_ERR_BAD_SHAPE;
     if (R > INT32_MAX - 64 || H > (INT32_MAX - 1024) / 2) return TK_ERR_TOO_LARGE;
+    if (2 * H * (x_dtype == TK_BF16 ? 2 : 4) > (int64_t)UINT32_MAX) return TK_ERR_TOO_LARGE;   // byte offsets inside a row are 32-bit
     if (group != 128 && group != H) return TK_ERR_BAD_GROUP;
     if (group != 128 && sf_layout != TK_SF_ROW_F32) return TK_ERR_BAD_LAYOUT;
     if (clamped_count && !use_clamp) return TK_ERR_BAD_MODE;
