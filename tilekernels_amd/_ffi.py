@@ -101,8 +101,32 @@ def ptr(t) -> int:
     return 0 if t is None else t.data_ptr()
 
 
+# torch's own accessor of the raw stream handle (what its compiled extensions use): no Stream object per call
+_raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+
+
 def current_stream(device: torch.device) -> int:
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _SameDevice:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_SAME_DEVICE = _SameDevice()
+
+
+def on_device(device: torch.device):
+    """Context in which `device` is the current one: a switch only where it is not already."""
+    if device.index is not None and device.index == torch.cuda.current_device():
+        return _SAME_DEVICE
+    return torch.cuda.device(device)
 
 
 def require_gpu(*tensors) -> torch.device:

@@ -20,7 +20,7 @@ def expand_to_fused(x: torch.Tensor, token_topk_to_pos: torch.Tensor, pos_to_exp
     lib = _ffi.load()
     out = torch.empty((num_expanded_tokens, hidden), dtype=x.dtype, device=dev)
     if num_tokens > 0:
-        with torch.cuda.device(dev):
+        with _ffi.on_device(dev):
             rc = lib.tk_expand_to_fused(x.data_ptr(), num_tokens, hidden * x.element_size(), token_topk_to_pos.data_ptr(), num_topk,
                                         pos_to_expert.data_ptr(), num_expanded_tokens, out.data_ptr(), 0, 0, 0, 0, 0,
                                         _ffi.current_stream(dev))
@@ -59,7 +59,7 @@ def expand_to_fused_with_sf(x: QuantTensor, num_per_channels: int, token_topk_to
     ld = shape[1]
     out_sf = out_sf[:, :num_expanded_tokens] if use_tma_aligned_col_major_sf else out_sf
     if num_tokens > 0:
-        with torch.cuda.device(dev):
+        with _ffi.on_device(dev):
             rc = lib.tk_expand_to_fused(x.data_ptr(), num_tokens, hidden * x.element_size(), token_topk_to_pos.data_ptr(), num_topk,
                                         pos_to_expert.data_ptr(), num_expanded_tokens, out.data_ptr(), x_sf.data_ptr(), hidden_sf,
                                         out_sf.data_ptr(), ld, int(use_tma_aligned_col_major_sf), _ffi.current_stream(dev))

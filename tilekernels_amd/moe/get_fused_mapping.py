@@ -36,7 +36,7 @@ def get_fused_mapping(topk_idx: torch.Tensor, num_experts: int, num_expanded_tok
     ws_bytes = lib.tk_fused_mapping_workspace_bytes(num_tokens, num_topk, num_experts)
     workspace = torch.empty((max(ws_bytes, 4) // 4,), **i32)
 
-    with torch.cuda.device(dev):
+    with _ffi.on_device(dev):
         rc = lib.tk_get_fused_mapping(
             topk_idx.data_ptr(), num_tokens, num_topk, num_experts, alignment, num_expanded_tokens,
             pos_to_expert.data_ptr(), pos_to_token.data_ptr(), pos_to_token_topk.data_ptr(), token_topk_to_pos.data_ptr(),

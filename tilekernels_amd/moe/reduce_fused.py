@@ -51,7 +51,7 @@ def reduce_fused(
     if num_tokens > 0:
         lib = _ffi.load()
         out_code = _ffi.TK_OUT_E4M3 if out_dtype == torch.float8_e4m3fn else _ffi.dtype_code(x)
-        with torch.cuda.device(dev):
+        with _ffi.on_device(dev):
             rc = lib.tk_reduce_fused(x.data_ptr(), _ffi.dtype_code(x), num_expanded_tokens, hidden, _ffi.ptr(x_sf), _ffi.ptr(topk_weights),
                                      token_topk_to_pos.data_ptr(), num_tokens, num_topk, out.data_ptr(), out_code, _ffi.ptr(sf),
                                      _ffi.current_stream(dev))

@@ -40,7 +40,7 @@ def cast_back(x: QuantTensor, fmt: str, x_block_size: tuple, x_special_fmt: Opti
     out = torch.empty((num_tokens, hidden), dtype=out_dtype, device=dev)
     if num_tokens > 0:
         store, layout, ld = _input_sf_storage(x_sf)
-        with torch.cuda.device(dev):
+        with _ffi.on_device(dev):
             rc = lib.tk_cast_back(data.data_ptr(), in_fmt, num_tokens, hidden,
                                   store.data_ptr(), ld, layout, x_block_size[0], x_block_size[1], out.data_ptr(),
                                   _ffi.TK_F32 if fmt == 'fp32' else _ffi.TK_BF16, _ffi.current_stream(dev))

@@ -87,7 +87,8 @@ def cast_epilogue(out_sf: torch.Tensor, num_tokens: int, hidden: int, config: Ca
             out_sf = out_sf.view(torch.int32)
     if config.use_tma_aligned_col_major_sf:
         out_sf = out_sf.T
-    return out_sf[: ceil_div(num_tokens, config.sf_block[0]), :]
+    rows = ceil_div(num_tokens, config.sf_block[0])
+    return out_sf if out_sf.shape[0] == rows else out_sf[:rows, :]
 
 
 def unpack_from_e2m1fn_x2(x: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:

@@ -37,7 +37,7 @@ def per_block_cast_impl(x, fmt, block_size, use_tma_aligned_col_major_sf=False, 
 
     if num_tokens > 0:
         mode = _ffi.TK_SF_ONLY if sf_only else (_ffi.TK_CAST_GIVEN_SF if sf is not None else _ffi.TK_CAST_AND_SF)
-        with torch.cuda.device(dev):
+        with _ffi.on_device(dev):
             rc = lib.tk_per_block_cast(
                 x.data_ptr(), _ffi.dtype_code(x), num_tokens, hidden, 0 if sf_only else out.data_ptr(),
                 out_sf.data_ptr(), sf_leading_dim(out_sf), out_config.fmt_code, bm, bk, out_config.layout_code,

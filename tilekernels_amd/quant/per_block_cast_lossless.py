@@ -37,7 +37,7 @@ def per_block_cast_lossless(
     out_sf = alloc_scaling_factors((num_tokens, hidden), out_config, dev)
     if num_tokens > 0:
         store, layout, ld = _input_sf_storage(x_sf)
-        with torch.cuda.device(dev):
+        with _ffi.on_device(dev):
             rc = lib.tk_per_block_cast_lossless(
                 data.data_ptr(), num_tokens, hidden, store.data_ptr(), ld, layout, x_block_size[0], x_block_size[1],
                 out.data_ptr(), out_sf.data_ptr(), sf_leading_dim(out_sf), out_config.layout_code,

@@ -21,7 +21,7 @@ def _launch(x, x_sf, num_tokens, hidden, pos_to_token, num_tokens_out, num_per_t
     out = torch.empty(out_shape, dtype=torch.float8_e4m3fn, device=dev)
     out_sf = torch.empty((ceil_div(num_tokens_out, num_per_tokens), hidden), dtype=torch.float32, device=dev)
     if num_tokens_out > 0:
-        with torch.cuda.device(dev):
+        with _ffi.on_device(dev):
             rc = lib.tk_per_channel_cast(
                 x.data_ptr(), _ffi.TK_F32 if x.dtype == torch.float32 else _ffi.TK_BF16, _ffi.ptr(x_sf), num_tokens, hidden, _ffi.ptr(pos_to_token), num_tokens_out,
                 out.data_ptr(), out_sf.data_ptr(), num_per_tokens, int(round_sf), int(transpose), int(swiglu),

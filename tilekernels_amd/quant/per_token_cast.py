@@ -48,7 +48,7 @@ def per_token_cast_impl(x, fmt, num_per_channels, x_block_size=None, use_tma_ali
 
     if num_tokens > 0:
         mode = _ffi.TK_SF_ONLY if sf_only else (_ffi.TK_CAST_GIVEN_SF if sf is not None else _ffi.TK_CAST_AND_SF)
-        with torch.cuda.device(dev):
+        with _ffi.on_device(dev):
             rc = lib.tk_per_token_cast(
                 x.data_ptr(), _ffi.dtype_code(x), num_tokens, hidden, x.stride(0) if num_tokens > 1 else hidden,
                 0 if sf_only else out.data_ptr(), out_sf.data_ptr(), sf_leading_dim(out_sf),
@@ -101,7 +101,7 @@ def _per_token_cast_quantised_input(x, fmt, num_per_channels, x_block_size, use_
     out_sf = alloc_scaling_factors((num_tokens, hidden), out_config, dev)
     if num_tokens > 0:
         store, layout, ld = _input_sf_storage(x_sf)
-        with torch.cuda.device(dev):
+        with _ffi.on_device(dev):
             rc = lib.tk_per_token_cast_quantized(
                 data.data_ptr(), _ffi.TK_E2M1 if in_fp4 else _ffi.TK_E4M3, num_tokens, hidden, token_stride,
                 store.data_ptr(), ld, layout, x_block_size[0], x_block_size[1],

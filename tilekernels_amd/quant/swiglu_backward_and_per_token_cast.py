@@ -64,7 +64,7 @@ def swiglu_backward_and_per_token_cast(
 
     # also launched without rows: weight_grad of unrouted pairs is still defined (zero)
     if num_expand_tokens > 0 or weight.numel() > 0:
-        with torch.cuda.device(dev):
+        with _ffi.on_device(dev):
             rc = lib.tk_swiglu_backward_per_token_cast(
                 x.data_ptr(), x_sf.data_ptr(), num_expand_tokens, hidden, num_per_channels, grad_out.data_ptr(),
                 weight.data_ptr(), pos_to_token_topk.data_ptr(), token_topk_to_pos.data_ptr(), weight.numel(),

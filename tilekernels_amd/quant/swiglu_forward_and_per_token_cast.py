@@ -65,7 +65,7 @@ def swiglu_forward_and_per_token_cast(
     out = torch.empty((num_expanded_tokens, hidden), dtype=torch.float8_e4m3fn, device=dev)
     out_sf = alloc_scaling_factors((num_expanded_tokens, hidden), out_config, dev)
     if num_expanded_tokens > 0:
-        with torch.cuda.device(dev):
+        with _ffi.on_device(dev):
             # the counting variant: at most 8 workgroups per compute unit, which then loop over tiles (every workgroup that
             # clamped anything sends one atomic request to the counters, and those are served one at a time)
             max_blocks = get_num_sms() * 8 if clamped_count is not None else 0
