@@ -404,3 +404,36 @@ def test_swiglu_cast_variants_match_the_product(spec):
     torch.cuda.synchronize()
     assert torch.equal(out, codes.view(torch.uint8)), 'codes'
     assert torch.equal(out_sf, sf), 'scales'
+
+
+def test_smallest_shapes():
+    """One to three rows of one or two groups: every lane but a few is beyond the data."""
+    tk, f = _tk(), Failures()
+    for N, layout, groups, M, fmt, dtype in itertools.product([16, 32, 64, 128], [LAYOUTS[0], LAYOUTS[2], LAYOUTS[4]], [1, 2], [1, 2, 3],
+                                                              ['e4m3', 'e2m1'], [torch.bfloat16, torch.float32]):
+        K = N * groups
+        kw = _kw(layout)
+        x = _randn((M, K), dtype, N + K + M, 2.0)
+        want = torch_ref.cast(x, fmt, (1, N), **kw)
+
+        def token():
+            got = tk.quant.per_token_cast(x.cuda(), fmt, N, **kw)
+            assert_same(got[0], want[0], 'codes')
+            assert_same(got[1], want[1], 'sf')
+            if K % 64 == 0:     # (dequantisation takes rows of a multiple of 64 elements, like the reference's)
+                assert_same(tk.quant.cast_back(got, 'fp32', (1, N)), torch_ref.cast_back(want, 'fp32', (1, N)), 'values')
+
+        f.run(f'per-token M={M} K={K} N={N} {fmt} {layout}', token)
+    for blk, (M, K), fmt in itertools.product([(128, 128), (32, 32)], [(1, 64), (2, 128), (3, 192)], ['e4m3', 'e2m1']):
+        x = _randn((M, K), torch.bfloat16, M + K, 2.0)
+        want = torch_ref.cast(x, fmt, blk)
+
+        def block():
+            got = tk.quant.per_block_cast(x.cuda(), fmt, blk)
+            assert_same(got[0], want[0], 'codes')
+            assert_same(got[1], want[1], 'sf')
+
+        f.run(f'per-block M={M} K={K} {blk} {fmt}', block)
+    for R, H, layout in itertools.product([1, 2, 3], [128, 256], [LAYOUTS[0], LAYOUTS[2], LAYOUTS[4]]):
+        f.run(f'swiglu R={R} H={H} {layout}', lambda: _swiglu_case(tk, torch.bfloat16, R, H, 128, layout, False, False, 0, R + H))
+    f.check(300)
