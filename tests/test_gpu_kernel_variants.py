@@ -82,11 +82,29 @@ def test_per_token_cast_variants(dtype, fmt):
             expect = torch_ref.cast(x, fmt, (1, N), sf=want[1], **kw)
             assert_same(tk.quant.per_token_cast_with_precomputed_sf(xd, fmt, N, want[1].cuda(), **kw), expect, 'codes for given sf')
 
+        def strided():
+            # rows 16 bytes further apart than they are long; given scales in rows with three unused words behind them
+            wide = torch.zeros((M, K + 16 // x.element_size()), dtype=dtype, device='cuda')
+            view = wide[:, :K]
+            view.copy_(xd)
+            got = tk.quant.per_token_cast(view, fmt, N, **kw)
+            assert_same(got[0], want[0], 'codes of strided rows')
+            assert_same(got[1], want[1], 'sf of strided rows')
+            assert_same(tk.quant.per_token_cast_with_sf_only(view, fmt, N, **kw), want[1], 'sf alone of strided rows')
+            if not layout[0]:
+                sf_wide = torch.zeros((M, K // N + 3), dtype=torch.float32, device='cuda')
+                sf_view = sf_wide[:, :K // N]
+                sf_view.copy_(want[1].cuda())
+                expect = torch_ref.cast(x, fmt, (1, N), sf=want[1], **kw)
+                assert_same(tk.quant.per_token_cast_with_precomputed_sf(view, fmt, N, sf_view, **kw), expect, 'codes for given strided sf')
+
         desc = f'M={M} K={K} N={N} {layout}'
         f.run(desc, full)
         f.run(desc + ' sf only', only)
         if not layout[0]:
             f.run(desc + ' given sf', given)
+        if layout in (LAYOUTS[0], LAYOUTS[4]):
+            f.run(desc + ' strided', strided)
     f.check(500)
 
 
