@@ -455,3 +455,24 @@ def test_smallest_shapes():
     for R, H, layout in itertools.product([1, 2, 3], [128, 256], [LAYOUTS[0], LAYOUTS[2], LAYOUTS[4]]):
         f.run(f'swiglu R={R} H={H} {layout}', lambda: _swiglu_case(tk, torch.bfloat16, R, H, 128, layout, False, False, 0, R + H))
     f.check(300)
+
+
+@pytest.mark.parametrize('fmt', ['e4m3', 'e2m1'])
+def test_per_block_cast_into_a_buffer_that_is_only_8_byte_aligned(fmt):
+    """The wide tiles of mid-sized matrices store 16 codes per lane; the entry point only asks for 8-byte alignment of the codes."""
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    M, K = 4096, 2048
+    x = _randn((M, K), torch.bfloat16, 17, 2.0)
+    want = torch_ref.cast(x, fmt, (128, 128))
+    nbytes = want[0].numel()
+    buf = torch.full((nbytes + 32,), 0x5A, dtype=torch.uint8, device='cuda')
+    sf = torch.empty((M // 128, K // 128), dtype=torch.float32, device='cuda')
+    xd = x.cuda()
+    rc = lib.tk_per_block_cast(xd.data_ptr(), 0, M, K, buf.data_ptr() + 8, sf.data_ptr(), K // 128, 0 if fmt == 'e4m3' else 1, 128, 128, 0, 0, 0,
+                               torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    assert torch.equal(buf[8:8 + nbytes].cpu(), want[0].view(torch.uint8).flatten()), 'codes'
+    assert bool((buf[:8] == 0x5A).all()) and bool((buf[8 + nbytes:] == 0x5A).all()), 'bytes around the codes were written'
+    assert_same(sf, want[1], 'sf')
