@@ -58,7 +58,9 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_bac
                 // scale, and writes nothing
                 const bool ok = (FULL || c < K) && (FULL || row0 + r < M);
                 raw[r][h].load(ok ? elem_ptr<InT>(x, row0 + r, K, c) : x);
+                vmem_issue_gap();
                 raw[r][h].s = sf_load(sf, ok ? (row0 + r) / bm : 0, ok ? c / bk : 0);
+                vmem_issue_gap();
             }
         }
 #pragma unroll
@@ -80,7 +82,9 @@ __global__ __launch_bounds__(WIDE ? 64 * kMaxWideWaves : kThreads) void cast_bac
         for (int r = 0; r < RPW; ++r) {
             const bool ok = col_ok && (FULL || row0 + r < M);
             raw[r].load(ok ? elem_ptr<InT>(x, row0 + r, K, col) : x);
+            vmem_issue_gap();
             raw[r].s = sf_load(sf, ok ? (row0 + r) / bm : 0, ok ? col / bk : 0);
+            vmem_issue_gap();
         }
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
@@ -130,7 +134,9 @@ __global__ __launch_bounds__(kThreads) void cast_back_flat_kernel(const void *x,
                 row[h] = (int)q;
                 col[h] = (int)rem * 8;
                 raw[h].load(ok[h] ? elem_ptr<InT>(x, row[h], K, col[h]) : x);
+                vmem_issue_gap();
                 raw[h].s = sf_load(sf, ok[h] ? blk_m(row[h]) : 0, ok[h] ? blk_k(col[h]) : 0);
+                vmem_issue_gap();
             }
 #pragma unroll
             for (int h = 0; h < 2; ++h) {

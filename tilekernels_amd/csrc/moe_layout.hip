@@ -429,7 +429,7 @@ constexpr int kReduceUnroll = 8;
 struct SplitF32 {};
 struct Raw8SplitF32 {
     u32x4 a, b;
-    __device__ __forceinline__ void load(const float *p) { a = ld_stream16(p); b = ld_stream16(p + 256); }
+    __device__ __forceinline__ void load(const float *p) { a = ld_stream16(p); vmem_issue_gap(); b = ld_stream16(p + 256); }
     __device__ __forceinline__ void get(float (&v)[8]) const {
         v[0] = u2f(a.x); v[1] = u2f(a.y); v[2] = u2f(a.z); v[3] = u2f(a.w);
         v[4] = u2f(b.x); v[5] = u2f(b.y); v[6] = u2f(b.z); v[7] = u2f(b.w);
@@ -455,6 +455,7 @@ __device__ __forceinline__ void reduce_terms(float (&acc)[8], const typename Red
         // a skipped term reads row 0 (no branch around the loads) and is not added
         const int row = live[j] ? p : 0;
         raw[j].load(x + (int64_t)row * hidden + col);
+        vmem_issue_gap();
         s[j] = 1.0f;
         if (topk_weights) s[j] = live[j] ? uniform_load(topk_weights + (int64_t)t * num_topk + k) : 0.0f;
         if (x_sf) s[j] = s[j] * uniform_load(x_sf + row);

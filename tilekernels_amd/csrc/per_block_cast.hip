@@ -69,6 +69,7 @@ __device__ __forceinline__ void per_block_cast_tile(const PerBlockParams &p) {
     for (int i = 0; i < NI; ++i) {
         if (FULL) raw[i].template load_run<RUN>(x + (int64_t)(TR * i) * p.K, c % RUN);
         else raw[i].load(x + (int64_t)(TR * i) * p.K, col_ok && row0 + TR * i < p.M);
+        if (i + 1 < NI) vmem_issue_gap();
     }
     if constexpr (FULL && XB != 0) {
 #pragma unroll

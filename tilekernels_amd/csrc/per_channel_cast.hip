@@ -127,7 +127,9 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
             for (int r = 0; r < kPcRows; ++r) {
                 const uint16_t *xr = reinterpret_cast<const uint16_t *>(p.x) + (int64_t)(tok0 + r) * in_ld + col;
                 rg[r].load(xr);
+                vmem_issue_gap();
                 ru[r].load(xr + p.K);
+                vmem_issue_gap();
             }
             __builtin_amdgcn_sched_barrier(0);
             // the clamp arguments lie beyond the preloaded ones: touched only now, behind the loads.
@@ -163,13 +165,17 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
                 }
                 if constexpr (MODE == PC_E4M3) {
                     raw[r].load(reinterpret_cast<const uint8_t *>(p.x) + (int64_t)src * in_ld + col);
+                    vmem_issue_gap();
                     raw[r].s = p.x_sf[(int64_t)src * (p.K >> 7) + (col >> 7)];
+                    vmem_issue_gap();
                     if (GATHER && !valid) raw[r].zero();
                 } else if constexpr (MODE == PC_F32) {
                     raw[r].load(reinterpret_cast<const float *>(p.x) + (int64_t)src * in_ld + col);
+                    vmem_issue_gap();
                     if (GATHER && !valid) raw[r].zero();
                 } else {
                     raw[r].load(reinterpret_cast<const uint16_t *>(p.x) + (int64_t)src * in_ld + col);
+                    vmem_issue_gap();
                     if (GATHER && !valid) raw[r].zero();
                 }
             }
@@ -318,6 +324,7 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_fp8in_kernel(T
                 src = valid ? src : 0;
             }
             const u32x4 w = ld_stream16(reinterpret_cast<const uint8_t *>(p.x) + (int64_t)src * p.K + col);
+            vmem_issue_gap();
             lo[r].w = u32x2{w.x, w.y};
             hi[r].w = u32x2{w.z, w.w};
             lo[r].s = hi[r].s = p.x_sf[(int64_t)src * (p.K >> 7) + (col >> 7)];

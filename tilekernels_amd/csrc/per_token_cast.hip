@@ -112,6 +112,7 @@ __global__ __launch_bounds__(TILE == T_WIDE ? 64 * kMaxWideWaves : kThreads) voi
             raw[r].load(ok ? xp : p.x);
             if (!ok) raw[r].zero();
         }
+        if (r + 1 < RPW) vmem_issue_gap();
         if constexpr (Elem<InT>::quantised) {
             // the 8 codes of a lane share one input scale (input blocks are at least 32 columns wide)
             const bool ok = col_ok && (FULL || row0 + r < p.M);
@@ -209,6 +210,7 @@ __global__ __launch_bounds__(kThreads) void per_token_cast_q16_kernel(TK_PT_KERN
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
         const u32x4 w = ld_stream16(elem_ptr<e4m3in_t>(p.x, row0, p.x_ld, col + r * kWide));
+        if (r + 1 < RPW) vmem_issue_gap();
         lo[r].w = u32x2{w.x, w.y};
         hi[r].w = u32x2{w.z, w.w};
         lo[r].s = hi[r].s = sf_load(p.xsf, row0 / p.in_bm, (col + r * kWide) / p.in_bk);
@@ -273,6 +275,7 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERN
             // a lane beyond the end of the row reads the row's first elements (no branch around the loads)
             const int col = (i * nt + threadIdx.x) * 8;
             held[i].load(x + ((EXACT || col < p.K) ? col : 0));
+            if (i + 1 < ITER) vmem_issue_gap();
         }
 #pragma unroll
         for (int i = 0; i < ITER; ++i) {
@@ -390,6 +393,7 @@ __global__ __launch_bounds__(kThreads) void per_token_cast_flat_kernel(TK_PT_KER
         ok[r] = row[r] < p.M && col < p.K;
         // no branch around the load: a lane beyond the matrix reads its first bytes and is cleared by value
         raw[r].load(ok[r] ? elem_ptr<InT>(p.x, row[r], p.x_ld, col) : p.x);
+        if (r + 1 < RPW) vmem_issue_gap();
         if (!ok[r]) raw[r].zero();
     }
 

@@ -36,7 +36,9 @@ __global__ __launch_bounds__(kThreads) void stream_floor_kernel(const bf16_t *x,
 #pragma unroll
     for (int r = 0; r < PIECES; ++r) {
         a[r] = ld_stream16(src + r * kStripCols);
+        vmem_issue_gap();
         b[r] = TWO ? ld_stream16(src + cols + r * kStripCols) : u32x4{0u, 0u, 0u, 0u};
+        if (TWO) vmem_issue_gap();
     }
     if constexpr (STAMP) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -95,7 +97,9 @@ __global__ __launch_bounds__(kThreads) void stream_floor_tailed_kernel(const bf1
     for (int r = 0; r < 4; ++r) {
         if (r < np) {      // wave-uniform
             a[r] = ld_stream16(src + r * kStripCols);
+            vmem_issue_gap();
             b[r] = TWO ? ld_stream16(src + cols + r * kStripCols) : u32x4{0u, 0u, 0u, 0u};
+            if (TWO) vmem_issue_gap();
         }
     }
     uint32_t fold = 0;
@@ -134,6 +138,7 @@ __global__ __launch_bounds__(kThreads) void stream_floor_flat_kernel(const uint8
     for (int r = 0; r < PIECES; ++r) {
         const int64_t piece = first + r < pieces ? first + r : first;       // (a wave's surplus pieces read its first again)
         v[r] = floor_load<IN>(in + (piece * 64 + lane) * IN);
+        vmem_issue_gap();
     }
     uint32_t fold = 0;
 #pragma unroll

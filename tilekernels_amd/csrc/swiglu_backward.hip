@@ -90,8 +90,11 @@ __global__ __launch_bounds__(64 * kBwdMaxWaves) void swiglu_backward_kernel(TK_B
             const int64_t row = row0 + r;
             const uint8_t *xr = x + row * (2 * (int64_t)H) + col;
             rg[r].load(xr, ok);
+            vmem_issue_gap();
             ru[r].load(xr + H, ok);
+            vmem_issue_gap();
             rgo[r].load(grad_out + row * (int64_t)H + col, ok);
+            vmem_issue_gap();
             rg[r].s = ok ? x_sf[row * nsf + grp] : 0.0f;
             ru[r].s = ok ? x_sf[row * nsf + hsf + grp] : 0.0f;
         }

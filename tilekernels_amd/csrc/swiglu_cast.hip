@@ -199,7 +199,9 @@ __device__ __forceinline__ void swiglu_row_wave(SwigluParams p, int row0, int st
     for (int r = 0; r < NP; ++r) {
         const uint8_t *xg = xrow + (uint64_t)r * (uint64_t)rstep * sizeof(InT) + (uint32_t)(r * cstep) * (uint32_t)sizeof(InT);
         rg[r].load(xg + lane_off);
+        vmem_issue_gap();
         ru[r].load(xg + uh * (uint32_t)sizeof(InT) + lane_off);
+        if (r + 1 < NP) vmem_issue_gap();
     }
     fetch_late_arguments(p, CLAMP != 0, WEIGHTED, SF != 0);
     float w[NP];
@@ -413,13 +415,17 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
                                     (uint32_t)(r * kColStep) * (uint32_t)sizeof(InT);
                 const uint32_t lane_off = (uint32_t)strip * (uint32_t)(kStripCols * sizeof(InT)) + (uint32_t)lane * (uint32_t)(8 * sizeof(InT));
                 rg[r].template load_run<64>(xg + lane_off, lane);
+                vmem_issue_gap();
                 ru[r].template load_run<64>(xg + uh * (uint32_t)sizeof(InT) + lane_off, lane);
+                if (r + 1 < RPW) vmem_issue_gap();
             } else if (FULL && XB != 0) {
                 // (a padding row reads the first 2 KB of the matrix, as one run)
                 const bool ok = live[r];
                 const InT *src = ok ? xr : reinterpret_cast<const InT *>(p.x) + lane * 8;
                 rg[r].template load_run<64>(src, lane);
+                vmem_issue_gap();
                 ru[r].template load_run<64>(ok ? xr + uh : src, lane);
+                if (r + 1 < RPW) vmem_issue_gap();
                 if (!ok) { rg[r].zero(); ru[r].zero(); }
             } else {
                 // no branch around the loads (a branch would make the compiler wait for all eight loads
@@ -428,7 +434,9 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
                 const bool ok = live[r] && piece_ok;
                 const InT *src = ok ? xr : reinterpret_cast<const InT *>(p.x);
                 rg[r].load(src);
+                vmem_issue_gap();
                 ru[r].load(ok ? xr + uh : src);
+                if (r + 1 < RPW) vmem_issue_gap();
                 if (!ok) { rg[r].zero(); ru[r].zero(); }
             }
         }

@@ -95,13 +95,17 @@ __global__ __launch_bounds__(64 * kMaxWideWaves) void swiglu_variant_kernel(cons
 #pragma unroll
         for (int r = 0; r < AHEAD && r < RPW; ++r) {
             gw[r] = ld_stream16(xr + r * kStripCols);
+            vmem_issue_gap();
             uw[r] = ld_stream16(xr + H + r * kStripCols);
+            vmem_issue_gap();
         }
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
             if (r + AHEAD < RPW) {
                 gw[r + AHEAD < RPW ? r + AHEAD : 0] = ld_stream16(xr + (r + AHEAD) * kStripCols);
+                vmem_issue_gap();
                 uw[r + AHEAD < RPW ? r + AHEAD : 0] = ld_stream16(xr + H + (r + AHEAD) * kStripCols);
+                vmem_issue_gap();
             }
             float v[8];
             eval_piece<false>(gw[r], uw[r], v);
@@ -117,7 +121,9 @@ __global__ __launch_bounds__(64 * kMaxWideWaves) void swiglu_variant_kernel(cons
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
         gw[r] = ld_stream16(xr + r * kStripCols);
+        vmem_issue_gap();
         uw[r] = ld_stream16(xr + H + r * kStripCols);
+        vmem_issue_gap();
     }
     if constexpr (VARIANT == V_PRIO) asm volatile("s_waitcnt vmcnt(%0)\n\ts_setprio 3" ::"n"(2 * RPW - 1) : "memory");
     bool piecewise = VARIANT == V_PIECESF;
@@ -183,7 +189,9 @@ __global__ __launch_bounds__(kThreads) void swiglu_tail_kernel(const bf16_t *x, 
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             gw[r] = ld_stream16(xr + r * kStripCols);
+            vmem_issue_gap();
             uw[r] = ld_stream16(xr + H + r * kStripCols);
+            vmem_issue_gap();
         }
         float v[4][8], amax[4];
 #pragma unroll
@@ -200,7 +208,9 @@ __global__ __launch_bounds__(kThreads) void swiglu_tail_kernel(const bf16_t *x, 
         const int row = big * kWaves + (wg - big);
         const int col = wave * kStripCols + lane * 8;
         const bf16_t *xr = x + (int64_t)row * (2 * H) + col;
-        const u32x4 gw = ld_stream16(xr), uw = ld_stream16(xr + H);
+        const u32x4 gw = ld_stream16(xr);
+        vmem_issue_gap();
+        const u32x4 uw = ld_stream16(xr + H);
         float v[8];
         eval_piece<false>(gw, uw, v);
         const float inv = own_scale_store(group_allmax<16>(absmax8(v)), floor_, sf + (int64_t)row * (H / 128), wave * GPS + (lane >> 4), lane);

@@ -100,6 +100,22 @@ template <typename T> __device__ __forceinline__ T uniform_load(const T *p) {
 //     non-temporal loads, write-through stores 13.8 us   <- used here
 // Loads carry the `nt` bit; stores are issued at system scope (`sc0 sc1`), which writes them
 // through instead of leaving dirty lines to be flushed when the kernel ends.
+// Between two vector memory instructions of a wave that follow each other directly: one wait state.  A wave that issues its
+// loads back to back is served worse than one with anything at all between them (MI355X, the loads and stores of the fused
+// SwiGLU cast of bf16 [8192, 2 x 2048] alone, eight 16-byte loads per lane: back to back 14.07 us, one s_nop 0 / s_nop 3 /
+// s_nop 7 / 16 / 32 / 64 wait states between them 13.76 / 13.73 / 13.75 / 13.79 / 13.87 / 13.97; the order of the loads makes
+// no difference; the operator itself 14.05 -> 13.85 us; the same between stores changes nothing).  The compiler packs loads
+// whose addresses are ready together, so the gap is part of the text; the memory clobber keeps the loads on either side
+// where they are.
+#ifndef TK_VMEM_GAP
+#define TK_VMEM_GAP 1
+#endif
+__device__ __forceinline__ void vmem_issue_gap() {
+#if TK_VMEM_GAP
+    asm volatile("s_nop 0" ::: "memory");
+#endif
+}
+
 __device__ __forceinline__ u32x4 ld_stream16(const void *p) {
     return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
 }
@@ -152,7 +168,7 @@ template <> struct Raw8<bf16_t> {
 template <> struct Raw8<float> {
     u32x4 a, b;
     static constexpr int kXchgBytes = 32;   // LDS bytes per lane of a run
-    __device__ __forceinline__ void load(const void *p) { a = ld_stream16(p); b = ld_stream16(reinterpret_cast<const float *>(p) + 4); }
+    __device__ __forceinline__ void load(const void *p) { a = ld_stream16(p); vmem_issue_gap(); b = ld_stream16(reinterpret_cast<const float *>(p) + 4); }
     __device__ __forceinline__ void load(const void *p, bool ok) {
         zero();
         if (ok) load(p);
@@ -161,6 +177,7 @@ template <> struct Raw8<float> {
     template <int LANES> __device__ __forceinline__ void load_run(const void *p, int i) {
         const uint8_t *q = reinterpret_cast<const uint8_t *>(p) - 16 * i;
         a = ld_stream16(q);
+        vmem_issue_gap();
         b = ld_stream16(q + 16 * LANES);
     }
     // run_lds: the 32 * LANES bytes of LDS of this lane's run, 16-byte aligned
