@@ -30,20 +30,23 @@ __global__ __launch_bounds__(kThreads) void stream_floor_kernel(const bf16_t *x,
     const int row = tile_m * kWaves + wave;
     if (row >= rows) return;
     const int col = tile_k * PIECES * kStripCols + lane * 8;
-    const int64_t ld = (int64_t)cols * (TWO ? 2 : 1);
-    const bf16_t *src = x + row * ld + col;
+    // addresses as the operators form them: a wave-uniform base plus a 32-bit byte offset per lane
+    const uint32_t ucols = (uint32_t)cols;
+    const uint8_t *xrow = reinterpret_cast<const uint8_t *>(x) + (uint64_t)(uint32_t)row * ((TWO ? 4u : 2u) * ucols);
+    const uint32_t lane_off = (uint32_t)(tile_k * PIECES) * (uint32_t)(kStripCols * 2) + (uint32_t)lane * 16u;
+    const uint8_t *xup = xrow + ucols * 2u;      // the second half of the row
+    asm volatile("" : "+s"(xup));                // (kept in scalar registers)
     u32x4 a[PIECES], b[PIECES];
 #pragma unroll
     for (int r = 0; r < PIECES; ++r) {
-        a[r] = ld_stream16(src + r * kStripCols);
+        a[r] = ld_stream16(xrow + lane_off + r * (kStripCols * 2));
         vmem_issue_gap();
-        b[r] = TWO ? ld_stream16(src + cols + r * kStripCols) : u32x4{0u, 0u, 0u, 0u};
+        b[r] = TWO ? ld_stream16(xup + lane_off + r * (kStripCols * 2)) : u32x4{0u, 0u, 0u, 0u};
         if (TWO) vmem_issue_gap();
     }
-    if constexpr (STAMP) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        t_loaded = wall_clock64();
-    }
+    // every load is back before the first store goes out, as in the operators, whose stores follow all their arithmetic
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (STAMP) t_loaded = wall_clock64();
     uint32_t fold = 0;
 #pragma unroll
     for (int r = 0; r < PIECES; ++r) {
@@ -90,18 +93,23 @@ __global__ __launch_bounds__(kThreads) void stream_floor_tailed_kernel(const bf1
     }
     if (row >= rows) return;
     const int col = strip * kStripCols + lane * 8;
-    const int64_t ld = (int64_t)cols * (TWO ? 2 : 1);
-    const bf16_t *src = x + row * ld + col;
+    // (addresses as in stream_floor_kernel)
+    const uint32_t ucols = (uint32_t)cols;
+    const uint8_t *xrow = reinterpret_cast<const uint8_t *>(x) + (uint64_t)(uint32_t)row * ((TWO ? 4u : 2u) * ucols);
+    const uint8_t *xup = xrow + ucols * 2u;
+    asm volatile("" : "+s"(xup));
+    const uint32_t lane_off = (uint32_t)strip * (uint32_t)(kStripCols * 2) + (uint32_t)lane * 16u;
     u32x4 a[4], b[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         if (r < np) {      // wave-uniform
-            a[r] = ld_stream16(src + r * kStripCols);
+            a[r] = ld_stream16(xrow + lane_off + r * (kStripCols * 2));
             vmem_issue_gap();
-            b[r] = TWO ? ld_stream16(src + cols + r * kStripCols) : u32x4{0u, 0u, 0u, 0u};
+            b[r] = TWO ? ld_stream16(xup + lane_off + r * (kStripCols * 2)) : u32x4{0u, 0u, 0u, 0u};
             if (TWO) vmem_issue_gap();
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // (as in stream_floor_kernel)
     uint32_t fold = 0;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -140,6 +148,7 @@ __global__ __launch_bounds__(kThreads) void stream_floor_flat_kernel(const uint8
         v[r] = floor_load<IN>(in + (piece * 64 + lane) * IN);
         vmem_issue_gap();
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // (as in stream_floor_kernel)
     uint32_t fold = 0;
 #pragma unroll
     for (int r = 0; r < PIECES; ++r) {
@@ -195,7 +204,7 @@ extern "C" int tk_stream_floor_flat(const void *in, int64_t in_bytes, int in_byt
 static int stream_floor_launch(const void *x, int64_t rows, int64_t cols, int two_halves, void *out, void *sf, void *stamps,
                                bool stamp, void *stream) {
     if (rows < 0 || cols <= 0 || cols % 1024 != 0) return TK_ERR_BAD_SHAPE;
-    if (rows > INT32_MAX - 64 || cols > (INT32_MAX - 1024) / 2) return TK_ERR_TOO_LARGE;
+    if (rows > INT32_MAX - 64 || cols > (INT32_MAX - 1024) / 4) return TK_ERR_TOO_LARGE;      // (a row's bytes are counted in 32 bits)
     if (rows == 0) return TK_OK;
     if (!x || !out || (stamp && !stamps)) return TK_ERR_NULL_POINTER;
     if (!aligned_to(x, 16) || !aligned_to(out, 8) || !aligned_to(sf, 4) || !aligned_to(stamps, 8)) return TK_ERR_MISALIGNED;
@@ -235,7 +244,7 @@ extern "C" int tk_stream_floor_tailed(const void *x, int64_t rows, int64_t cols,
     if (rows < 0 || cols <= 0 || cols % 2048 != 0 || rows % 4 != 0 || rows_two < 0 || rows_one < 0 || rows_two % 4 != 0 || rows_one % 4 != 0 ||
         rows_two + rows_one > rows)
         return TK_ERR_BAD_SHAPE;
-    if (rows > INT32_MAX / 8 || cols > (INT32_MAX - 1024) / 2) return TK_ERR_TOO_LARGE;
+    if (rows > INT32_MAX / 8 || cols > (INT32_MAX - 1024) / 4) return TK_ERR_TOO_LARGE;
     if (rows == 0) return TK_OK;
     if (!x || !out) return TK_ERR_NULL_POINTER;
     if (!aligned_to(x, 16) || !aligned_to(out, 8) || !aligned_to(sf, 4)) return TK_ERR_MISALIGNED;
