@@ -67,6 +67,7 @@ __global__ __launch_bounds__(kLlThreads) void lossless_fp4_to_fp8_kernel(const u
         const bool ok = col_ok && row < M;
         const int rr = ok ? row : row_first, cc = ok ? col : col_first;
         code[p] = __builtin_nontemporal_load(reinterpret_cast<const Codes *>(x + (((int64_t)rr * K + cc) >> 1)));
+        vmem_issue_gap();
         e_in[p] = (int)(f2u(sf_load_select(xsf, rr >> ibm_sh, cc >> ibk_sh)) >> 23);
         if (!ok) { code[p] = Codes{}; e_in[p] = 0; }
     }

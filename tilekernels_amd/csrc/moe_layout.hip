@@ -225,6 +225,7 @@ __global__ __launch_bounds__(64 * kSingleWaves) void fused_mapping_single_kernel
         for (int j = 0; j < U; ++j) {
             const int pi = p0 + j * nthreads + tid;
             w[j] = wide[pi < pairs ? pi : 0];
+            vmem_issue_gap();
         }
 #pragma unroll
         for (int j = 0; j < U; ++j) {
