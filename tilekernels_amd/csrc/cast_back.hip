@@ -116,55 +116,72 @@ __global__ __launch_bounds__(kThreads) void cast_back_flat_kernel(const void *x,
     const SfRef sf{a_sf, a_sf_ld, a_sf_layout, nm, nk};
     const int lane = threadIdx.x & 63, wave = wave_id();
     const unsigned total = (unsigned)M * (unsigned)ppr;
+    // All loads of the wave's slots go out before its first store: with a slot's store in front of the next slot's loads
+    // the compiler must keep that order (input and output may overlap for all it knows) and the wave has one slot's
+    // loads in flight at a time.
+    if constexpr (OUT_F32) {
+        const bool hi = lane & 1;
+        Raw8<InT> raw[RPW][2];
+        int row[RPW][2], col[RPW][2];
+        bool ok[RPW][2];
 #pragma unroll
-    for (int r = 0; r < RPW; ++r) {
-        const unsigned slot = (unsigned)((blockIdx.x * kWaves + wave) * RPW + r);
-        if constexpr (OUT_F32) {
-            const bool hi = lane & 1;
-            Raw8<InT> raw[2];
-            int row[2], col[2];
-            bool ok[2];
+        for (int r = 0; r < RPW; ++r) {
+            const unsigned slot = (unsigned)((blockIdx.x * kWaves + wave) * RPW + r);
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const unsigned piece = slot * 64u + (unsigned)(h * 32 + (lane >> 1));
-                ok[h] = piece < total;
+                ok[r][h] = piece < total;
                 // piece / ppr by multiplication: with floor(2^32 / ppr) the quotient comes out exact or one too small
                 unsigned q = __umulhi(piece, ppr_recip), rem = piece - q * (unsigned)ppr;
                 if (rem >= (unsigned)ppr) { ++q; rem -= (unsigned)ppr; }
-                row[h] = (int)q;
-                col[h] = (int)rem * 8;
-                raw[h].load(ok[h] ? elem_ptr<InT>(x, row[h], K, col[h]) : x);
+                row[r][h] = (int)q;
+                col[r][h] = (int)rem * 8;
+                raw[r][h].load(ok[r][h] ? elem_ptr<InT>(x, row[r][h], K, col[r][h]) : x);
                 vmem_issue_gap();
-                raw[h].s = sf_load(sf, ok[h] ? blk_m(row[h]) : 0, ok[h] ? blk_k(col[h]) : 0);
+                raw[r][h].s = sf_load(sf, ok[r][h] ? blk_m(row[r][h]) : 0, ok[r][h] ? blk_k(col[r][h]) : 0);
                 vmem_issue_gap();
             }
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                if (!ok[h]) continue;
+                if (!ok[r][h]) continue;
                 float v[4];
-                raw[h].get4(v, hi);
-                const int64_t idx = (int64_t)row[h] * K + col[h] + (hi ? 4 : 0);
+                raw[r][h].get4(v, hi);
+                const int64_t idx = (int64_t)row[r][h] * K + col[r][h] + (hi ? 4 : 0);
                 __builtin_nontemporal_store(u32x4{f2u(v[0]), f2u(v[1]), f2u(v[2]), f2u(v[3])},
                                             reinterpret_cast<u32x4 *>(reinterpret_cast<float *>(out) + idx));
             }
-        } else {
-            const unsigned piece = slot * 64u + (unsigned)lane;
-            const bool ok = piece < total;
+        }
+    } else {
+        Raw8<InT> raw[RPW];
+        int row[RPW], col[RPW];
+        bool ok[RPW];
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            const unsigned piece = (unsigned)((blockIdx.x * kWaves + wave) * RPW + r) * 64u + (unsigned)lane;
+            ok[r] = piece < total;
             unsigned q = __umulhi(piece, ppr_recip), rem = piece - q * (unsigned)ppr;
             if (rem >= (unsigned)ppr) { ++q; rem -= (unsigned)ppr; }
-            const int row = (int)q, col = (int)rem * 8;
-            Raw8<InT> raw;
-            raw.load(ok ? elem_ptr<InT>(x, row, K, col) : x);
-            raw.s = sf_load(sf, ok ? blk_m(row) : 0, ok ? blk_k(col) : 0);
-            if (!ok) continue;
+            row[r] = (int)q;
+            col[r] = (int)rem * 8;
+            raw[r].load(ok[r] ? elem_ptr<InT>(x, row[r], K, col[r]) : x);
+            vmem_issue_gap();
+            raw[r].s = sf_load(sf, ok[r] ? blk_m(row[r]) : 0, ok[r] ? blk_k(col[r]) : 0);
+            vmem_issue_gap();
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            if (!ok[r]) continue;
             float v[8];
-            raw.get(v);
+            raw[r].get(v);
             u32x4 w;
             w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[0], v[1]}), bf16x2));
             w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[2], v[3]}), bf16x2));
             w.z = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[4], v[5]}), bf16x2));
             w.w = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{v[6], v[7]}), bf16x2));
-            __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(out) + (int64_t)row * K + col));
+            __builtin_nontemporal_store(w, reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(out) + (int64_t)row[r] * K + col[r]));
         }
     }
 }
