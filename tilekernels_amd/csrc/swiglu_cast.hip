@@ -536,7 +536,10 @@ __global__ __launch_bounds__(kThreads) void swiglu_cast_flat_kernel(TK_SWIGLU_KE
     const InT *xb = reinterpret_cast<const InT *>(p.x);
     ClampCounter<CLAMP> counter;
 
-    int row[RPW], grp[RPW];
+    // Mask entries and weight indices of all slots are asked for first, then the data of all slots, then the weights: a
+    // load whose address hangs on a loaded value waits for every load issued before it, so with a slot's mask entry read
+    // behind the previous slot's data a wave had one slot's data in flight at a time ([32768, 2 x 768] bf16 22.3 us).
+    int row[RPW], grp[RPW], expert[RPW], wpos[RPW];
     bool inside[RPW], live[RPW];
     Raw8<InT> rg[RPW], ru[RPW];
 #pragma unroll
@@ -548,15 +551,45 @@ __global__ __launch_bounds__(kThreads) void swiglu_cast_flat_kernel(TK_SWIGLU_KE
         if (rem >= (unsigned)gpr) { ++q; rem -= (unsigned)gpr; }
         row[r] = (int)q;
         grp[r] = (int)rem;
+        inside[r] = row[r] < p.R && grp[r] * 128 + own * 8 < p.H;
+        expert[r] = 0;
+        wpos[r] = -1;
+    }
+    // (one branch per table with the loads of all slots inside: a value that is loaded on one side of a branch and set on the
+    // other is waited for before the branch ends)
+    if (p.pos_to_expert) {
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) expert[r] = p.pos_to_expert[row[r] < p.R ? row[r] : 0];      // (lanes beyond the last row read row 0's entry)
+    }
+    if (p.pos_to_token_topk) {
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) wpos[r] = p.pos_to_token_topk[row[r] < p.R ? row[r] : 0];
+    }
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
         const int col = grp[r] * 128 + own * 8;
-        inside[r] = row[r] < p.R && col < p.H;
-        live[r] = row[r] < p.R && (p.pos_to_expert == nullptr || p.pos_to_expert[row[r]] >= 0);
+        live[r] = row[r] < p.R && expert[r] >= 0;
         // no branch around the loads: a padding row, and a lane beyond the matrix, reads its first bytes and is cleared by value
         const bool ok = inside[r] && live[r];
         const InT *src = ok ? xb + (int64_t)row[r] * (2 * (int64_t)p.H) + col : xb;
         rg[r].load(src);
+        vmem_issue_gap();
         ru[r].load(ok ? src + p.H : src);
+        vmem_issue_gap();
         if (!ok) { rg[r].zero(); ru[r].zero(); }
+    }
+    float w[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) w[r] = 0.0f;
+    if (p.pos_to_token_topk) {
+        bool has[RPW];
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            has[r] = live[r] && wpos[r] >= 0 && wpos[r] < p.num_weights;
+            w[r] = p.topk_weights[has[r] ? wpos[r] : 0];
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) w[r] = has[r] ? w[r] : 0.0f;
     }
 
     float v[RPW][8], amax[RPW];
@@ -569,13 +602,8 @@ __global__ __launch_bounds__(kThreads) void swiglu_cast_flat_kernel(TK_SWIGLU_KE
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[r][i] = silu_mul<InT>(g[i], u[i]);
         if (p.pos_to_token_topk) {
-            float w = 0.0f;
-            if (live[r]) {
-                const int pos = p.pos_to_token_topk[row[r]];
-                if (pos >= 0 && pos < p.num_weights) w = p.topk_weights[pos];
-            }
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[r][i] = v[r][i] * w;
+            for (int i = 0; i < 8; ++i) v[r][i] = v[r][i] * w[r];
         }
         amax[r] = group_allmax<16>(absmax8(v[r]));
     }
