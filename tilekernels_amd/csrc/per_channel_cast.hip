@@ -154,30 +154,41 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_kernel(TK_PC_K
                 raw[r].w = u32x4{pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]), pack_bf16x2(a[4], a[5]), pack_bf16x2(a[6], a[7])};
             }
         } else {
+            // (the gather indices of all rows are asked for before the first row's data: a load whose address hangs on a loaded value
+            // waits for every load issued before it)
+            int gathered[kPcRows];
+            bool valid[kPcRows];
+            if constexpr (GATHER) {
+#pragma unroll
+                for (int r = 0; r < kPcRows; ++r) gathered[r] = p.pos_to_token[tok0 + r];
+            }
 #pragma unroll
             for (int r = 0; r < kPcRows; ++r) {
                 int src = tok0 + r;
-                bool valid = true;
+                valid[r] = true;
                 if constexpr (GATHER) {
-                    src = p.pos_to_token[tok0 + r];
-                    valid = src >= 0 && src < p.num_tokens;
-                    src = valid ? src : 0;
+                    src = gathered[r];
+                    valid[r] = src >= 0 && src < p.num_tokens;
+                    src = valid[r] ? src : 0;
                 }
                 if constexpr (MODE == PC_E4M3) {
                     raw[r].load(reinterpret_cast<const uint8_t *>(p.x) + (int64_t)src * in_ld + col);
                     vmem_issue_gap();
                     raw[r].s = p.x_sf[(int64_t)src * (p.K >> 7) + (col >> 7)];
                     vmem_issue_gap();
-                    if (GATHER && !valid) raw[r].zero();
                 } else if constexpr (MODE == PC_F32) {
                     raw[r].load(reinterpret_cast<const float *>(p.x) + (int64_t)src * in_ld + col);
                     vmem_issue_gap();
-                    if (GATHER && !valid) raw[r].zero();
                 } else {
                     raw[r].load(reinterpret_cast<const uint16_t *>(p.x) + (int64_t)src * in_ld + col);
                     vmem_issue_gap();
-                    if (GATHER && !valid) raw[r].zero();
                 }
+            }
+            // (rows without a source are cleared once all loads are out: clearing a register a load is still to fill means waiting for it)
+            if constexpr (GATHER) {
+#pragma unroll
+                for (int r = 0; r < kPcRows; ++r)
+                    if (!valid[r]) raw[r].zero();
             }
         }
     }
@@ -314,12 +325,18 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_fp8in_kernel(T
 #pragma unroll
     for (int r = 0; r < kPcRows; ++r) { lo[r].zero(); hi[r].zero(); }
     if (rows_ok && col_ok) {
+        // (gather indices of all rows first: see per_channel_cast_kernel)
+        int gathered[kPcRows];
+        if constexpr (GATHER) {
+#pragma unroll
+            for (int r = 0; r < kPcRows; ++r) gathered[r] = p.pos_to_token[tok0 + r];
+        }
 #pragma unroll
         for (int r = 0; r < kPcRows; ++r) {
             int src = tok0 + r;
             bool valid = true;
             if constexpr (GATHER) {
-                src = p.pos_to_token[tok0 + r];
+                src = gathered[r];
                 valid = src >= 0 && src < p.num_tokens;
                 src = valid ? src : 0;
             }
@@ -328,7 +345,13 @@ __global__ __launch_bounds__(kPcThreads, 4) void per_channel_cast_fp8in_kernel(T
             lo[r].w = u32x2{w.x, w.y};
             hi[r].w = u32x2{w.z, w.w};
             lo[r].s = hi[r].s = p.x_sf[(int64_t)src * (p.K >> 7) + (col >> 7)];
-            if (GATHER && !valid) { lo[r].zero(); hi[r].zero(); }
+            vmem_issue_gap();
+            gathered[r] = valid ? 1 : 0;
+        }
+        if constexpr (GATHER) {      // (cleared once all loads are out)
+#pragma unroll
+            for (int r = 0; r < kPcRows; ++r)
+                if (!gathered[r]) { lo[r].zero(); hi[r].zero(); }
         }
     }
 

@@ -277,6 +277,9 @@ __global__ __launch_bounds__(kThreads) void per_token_rowgroup_kernel(TK_PT_KERN
             held[i].load(x + ((EXACT || col < p.K) ? col : 0));
             if (i + 1 < ITER) vmem_issue_gap();
         }
+        // (all loads are out before the first piece is looked at: left to itself the compiler moves the first piece's arithmetic in
+        // front of the later loads where the row may end inside a piece, and the pieces then arrive one round trip after the other)
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < ITER; ++i) {
             const int col = (i * nt + threadIdx.x) * 8;
