@@ -103,20 +103,27 @@ __global__ __launch_bounds__(TILE == T_WIDE ? 64 * kMaxWideWaves : kThreads) voi
 #pragma unroll
     for (int r = 0; r < RPW; ++r) {
         const void *xp = elem_ptr<InT>(p.x, row0 + r * kRowStep, p.x_ld, col + r * kColStep);
-        if (FULL) {
-            raw[r].template load_run<64>(xp, lane);
-        } else {
-            // no branch around the load (the loads of the wave's rows then go out together): a lane beyond the last
-            // row or column reads the first bytes of the matrix and is cleared by value
-            const bool ok = col_ok && row0 + r < p.M;
-            raw[r].load(ok ? xp : p.x);
-            if (!ok) raw[r].zero();
-        }
+        // no branch around a load (the loads of the wave's rows then go out together): a lane beyond the last row or
+        // column reads the first bytes of the matrix, and the first scale, and is cleared by value once all loads are out
+        // (clearing a register that a load is still to fill means waiting for that load)
+        const bool ok = col_ok && (FULL || row0 + r < p.M);
+        if (FULL) raw[r].template load_run<64>(xp, lane);
+        else raw[r].load(ok ? xp : p.x);
         if (r + 1 < RPW) vmem_issue_gap();
         if constexpr (Elem<InT>::quantised) {
             // the 8 codes of a lane share one input scale (input blocks are at least 32 columns wide)
+            raw[r].s = sf_load(p.xsf, ok ? (row0 + r * kRowStep) / p.in_bm : 0, ok ? (col + r * kColStep) / p.in_bk : 0);
+            vmem_issue_gap();
+        }
+    }
+    if constexpr (!FULL || Elem<InT>::quantised) {
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
             const bool ok = col_ok && (FULL || row0 + r < p.M);
-            raw[r].s = ok ? sf_load(p.xsf, (row0 + r * kRowStep) / p.in_bm, (col + r * kColStep) / p.in_bk) : 0.0f;
+            if (!FULL && !ok) raw[r].zero();
+            if constexpr (Elem<InT>::quantised) {
+                if (!ok) raw[r].s = 0.0f;
+            }
         }
     }
 
