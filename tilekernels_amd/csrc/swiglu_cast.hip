@@ -643,7 +643,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_cast_flat_kernel(TK_SWIGLU_KE
 // One scale per row (group == H): a workgroup per row.  Rows of up to ITER * 2048 outputs (ITER = 1..4) are
 // evaluated once and held in registers between the amax and the conversion; ITER == 0 takes longer rows and
 // evaluates the activation twice (amax pass, then convert pass; the second read comes from L2).  Row-major scales
-// only.  Measured on MI355X, bf16 [16384, 2 x 4096]: 79.2 us in two passes (90.7 us with the clamp), 52 - 55 us held;
+// only.  Measured on MI355X, bf16 [16384, 2 x 4096]: 79.2 us in two passes (90.7 us with the clamp), 51.4 us held;
 // fp32: 150.7 -> 102.2 us.
 template <typename InT, int CLAMP, int ITER>
 __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KERNEL_ARGS) {
@@ -653,7 +653,8 @@ __global__ __launch_bounds__(kThreads) void swiglu_rowgroup_kernel(TK_SWIGLU_KER
     const int nt = p.nwaves * 64;   // threads of the workgroup: the fewest whole waves that cover a row in ITER pieces
     ClampCounter<CLAMP> counter;
     for (int row = blockIdx.x; row < p.R; row += gridDim.x) {
-        const bool live = p.pos_to_expert == nullptr || p.pos_to_expert[row] >= 0;
+        // (the row's entry comes through the scalar path: as a vector load it is waited for by every lane in front of the row's data)
+        const bool live = p.pos_to_expert == nullptr || uniform_load(p.pos_to_expert + row) >= 0;
         uint8_t *out_row = p.out + (int64_t)row * p.H;
         float *sf_row = reinterpret_cast<float *>(p.sf.base) + (int64_t)row * p.sf.ld;
         if (!live) {
