@@ -476,3 +476,35 @@ def test_per_block_cast_into_a_buffer_that_is_only_8_byte_aligned(fmt):
     assert torch.equal(buf[8:8 + nbytes].cpu(), want[0].view(torch.uint8).flatten()), 'codes'
     assert bool((buf[:8] == 0x5A).all()) and bool((buf[8 + nbytes:] == 0x5A).all()), 'bytes around the codes were written'
     assert_same(sf, want[1], 'sf')
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+def test_masked_swiglu_cast_into_a_buffer_that_is_only_8_byte_aligned(dtype):
+    """Padding rows of the row-wise kernel are written as 16-byte stores where the buffer allows it and as 8-byte stores
+    otherwise; both must give the zeros (and nothing around the buffer) that the wrapper's 256-byte-aligned tensors get."""
+    import tilekernels_amd as tk
+    from tilekernels_amd import _ffi
+    lib = _ffi.load()
+    R, H = 1031, 2048
+    g = torch.Generator().manual_seed(23)
+    x = (torch.randn((R, 2 * H), generator=g) * 2.0).to(dtype).cuda()
+    pos_to_expert = torch.randint(0, 4, (R,), generator=g).to(torch.int32)
+    pos_to_expert[5:77] = -1
+    pos_to_expert[torch.rand((R,), generator=g) < 0.3] = -1
+    pos_to_expert[-1] = -1
+    pos_to_expert = pos_to_expert.cuda()
+    want, want_sf = tk.quant.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, pos_to_expert=pos_to_expert)
+    dead = (pos_to_expert < 0).cpu()
+    assert bool((want.view(torch.uint8)[dead.cuda()] == 0).all()) and bool((want_sf[dead.cuda()] == 0).all())
+    assert bool((want_sf[(~dead).cuda()] > 0).all())
+    for shift in (8, 16):
+        buf = torch.full((R * H + 64,), 0x5A, dtype=torch.uint8, device='cuda')
+        sf = torch.full((R, H // 128), -1.0, dtype=torch.float32, device='cuda')
+        rc = lib.tk_swiglu_per_token_cast(x.data_ptr(), _ffi.dtype_code(x), R, H, buf.data_ptr() + shift, sf.data_ptr(), H // 128, 128,
+                                          _ffi.TK_SF_ROW_F32, 0, -1.0, None, None, 0, pos_to_expert.data_ptr(), 0, 0.0, None, 0,
+                                          torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+        torch.cuda.synchronize()
+        assert torch.equal(buf[shift:shift + R * H].view(R, H), want.view(torch.uint8)), f'codes at +{shift}'
+        assert bool((buf[:shift] == 0x5A).all()) and bool((buf[shift + R * H:] == 0x5A).all()), f'bytes around the codes were written at +{shift}'
+        assert torch.equal(sf, want_sf), f'scales at +{shift}'

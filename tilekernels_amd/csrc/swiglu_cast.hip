@@ -405,6 +405,28 @@ __global__ __launch_bounds__(TILE == T_ROW ? 64 * kMaxWideWaves : kThreads) void
         if constexpr (EARLY_WEIGHT) {
             if (has_weight && (FULL || row0 < p.R)) wpos = uniform_load(p.pos_to_token_topk + row0);
         }
+        // A wave whose row is padding writes the row's zeros and leaves: no loads, no arithmetic.  The zeros go out as
+        // non-temporal 16-byte stores that cover whole lines.  Measured on MI355X, bf16, us per call, padding rows flowing
+        // through the arithmetic as zeros / this way: configuration with runs of padding (32768 live rows of 47488, H = 2048)
+        // 59.5 / 58.8, every third row padding ([32768, 2 x 2048]) 40.6 / 39.6.  With the write-through stores of the live
+        // rows the runs cost 63.0 (16 bytes per lane) and 63.4 (8 bytes per lane), the scattered padding 38.4: a burst of
+        // such stores to one stretch of memory is served slowly, and the runs are the layout this operator is made for.
+        if constexpr (MASK && DIRECT && FULL) {
+            if (expert[0] < 0) {
+                uint8_t *piece = p.out + (int64_t)row0 * p.H + strip * kStripCols;
+                if (RPW % 2 == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0) {
+#pragma unroll
+                    for (int i = 0; i < RPW / 2; ++i)
+                        __builtin_nontemporal_store(u32x4{0u, 0u, 0u, 0u}, reinterpret_cast<u32x4 *>(piece + i * 1024 + lane * 16));
+                } else {
+#pragma unroll
+                    for (int r = 0; r < RPW; ++r) st_stream8(piece + r * kColStep + lane * 8, u32x2{0u, 0u});
+                }
+                if (lane < RPW * GPS) st_stream4(reinterpret_cast<float *>(p.sf.base) + (int64_t)row0 * p.sf.ld + strip * GPS + lane, 0u);
+                if constexpr (LOOP) continue;
+                else return;
+            }
+        }
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
             live[r] = (FULL || row0 + r * kRowStep < p.R) && expert[r] >= 0;
