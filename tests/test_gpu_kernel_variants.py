@@ -508,3 +508,25 @@ def test_masked_swiglu_cast_into_a_buffer_that_is_only_8_byte_aligned(dtype):
         assert torch.equal(buf[shift:shift + R * H].view(R, H), want.view(torch.uint8)), f'codes at +{shift}'
         assert bool((buf[:shift] == 0x5A).all()) and bool((buf[shift + R * H:] == 0x5A).all()), f'bytes around the codes were written at +{shift}'
         assert torch.equal(sf, want_sf), f'scales at +{shift}'
+
+
+@pytest.mark.parametrize('dtype,R,H', [(torch.bfloat16, 40003, 2048), (torch.bfloat16, 9001, 8192), (torch.float32, 17001, 2048)])
+def test_swiglu_cast_of_a_launch_that_refills_the_gpu_many_times(dtype, R, H):
+    """Launches of more than 3.5 times the GPU's wave slots run one-wave workgroups; rows are independent, so the result
+    must equal that of the same rows cast in pieces small enough for the other launch shapes (which the oracle tests cover)."""
+    import tilekernels_amd as tk
+    g = torch.Generator().manual_seed(R)
+    x = (torch.randn((R, 2 * H), generator=g) * 2.5).to(dtype).cuda()
+    ptt = torch.randint(-1, R, (R,), generator=g).to(torch.int32).cuda()
+    w = torch.rand((R // 8 + 1, 8), generator=g).cuda()
+    for kw in ({}, dict(swiglu_clamp_value=2.0), dict(round_sf=True)):
+        for weighted in (False, True):
+            args = (ptt, w) if weighted else ()
+            out, sf = tk.quant.swiglu_forward_and_per_token_cast(x, 'e4m3', 128, *args, **kw)
+            step = 2048
+            for r0 in range(0, R, step):
+                r1 = min(R, r0 + step)
+                part_args = (ptt[r0:r1].contiguous(), w) if weighted else ()
+                o, s = tk.quant.swiglu_forward_and_per_token_cast(x[r0:r1], 'e4m3', 128, *part_args, **kw)
+                assert torch.equal(out[r0:r1].view(torch.uint8), o.view(torch.uint8)), f'codes of rows {r0}..{r1} {kw} weighted={weighted}'
+                assert torch.equal(sf[r0:r1], s), f'scales of rows {r0}..{r1} {kw} weighted={weighted}'

@@ -778,8 +778,13 @@ template <typename InT, int CLAMP, int RPW, int TILE>
 static void launch_swiglu_tiled(SwigluParams &p, int max_blocks, hipStream_t stream) {
     // T_ROW, rows per workgroup (= waves), us per call at [8192, 4096] dense / [48128, 4096] with a third of the rows
     // masked: 1: 14.9 / 61.6, 2: 14.85 / 62.1, 4: 14.68 / 62.9, 8: 15.15 / 63.4.  A masked batch is better off with
-    // single-wave workgroups: a wave whose row is padding is done at once and frees its slot alone.
-    const int waves = TILE == T_ROW && p.pos_to_expert ? 1 : kWaves;
+    // single-wave workgroups: a wave whose row is padding is done at once and frees its slot alone.  So is a launch of more
+    // than 3.5 times the GPU's wave slots (beyond those that end in smaller waves, below), where the slots are refilled
+    // several times over and a wave that is done need not wait for the three others of its workgroup to be replaced
+    // (four waves / one, bf16: [47360, 2 x 2048] 73.6 / 72.5, [65536, 2 x 2048] 101.1 / 99.0, [16384, 2 x 8192] 100.5 / 98.4,
+    // [131072, 2 x 2048] 211.1 / 209.2; fp32: [16384, 2 x 2048] 48.4 / 47.4, [32768, 2 x 2048] 93.9 / 92.1).
+    const bool many_turns = CLAMP != 2 && (int64_t)p.R * (p.H / kStripCols) / RPW * 2 > wave_slots() * 7;
+    const int waves = TILE == T_ROW && (p.pos_to_expert || many_turns) ? 1 : kWaves;
     const int rows = TILE == T_ROW || TILE == T_ROWC ? waves : kWaves * RPW;
     const int cols = TILE == T_ROW || TILE == T_ROWC ? RPW * kStripCols : kStripCols;
     const int tiles_m = (p.R + rows - 1) / rows;
