@@ -530,3 +530,27 @@ def test_swiglu_cast_of_a_launch_that_refills_the_gpu_many_times(dtype, R, H):
                 o, s = tk.quant.swiglu_forward_and_per_token_cast(x[r0:r1], 'e4m3', 128, *part_args, **kw)
                 assert torch.equal(out[r0:r1].view(torch.uint8), o.view(torch.uint8)), f'codes of rows {r0}..{r1} {kw} weighted={weighted}'
                 assert torch.equal(sf[r0:r1], s), f'scales of rows {r0}..{r1} {kw} weighted={weighted}'
+
+
+@pytest.mark.parametrize('fmt', ['e4m3', 'e2m1'])
+@pytest.mark.parametrize('group', [16, 32, 64, 128])
+def test_per_token_cast_of_fp32_rows_beyond_one_grid_plane(fmt, group):
+    """fp32 input runs one-wave workgroups on the row-wise tiles, so only a grid that overhangs along z (more than 32768
+    row tiles, not a multiple of that) has workgroups beyond the last row.  Rows are independent: the result must equal
+    that of the same rows cast in launches of one grid plane (which the oracle tests cover), with computed and given scales."""
+    import tilekernels_amd as tk
+    M, K = 32768 + 3, 2048
+    g = torch.Generator().manual_seed(group)
+    x = (torch.randn((M, K), generator=g) * 3.0).cuda()
+    out, sf = tk.quant.per_token_cast(x, fmt, group)
+    given = tk.quant.per_token_cast_with_precomputed_sf(x, fmt, group, sf)
+    given = given[0] if isinstance(given, tuple) else given
+    step = 8192
+    for r0 in range(0, M, step):
+        r1 = min(M, r0 + step)
+        o, s = tk.quant.per_token_cast(x[r0:r1], fmt, group)
+        assert torch.equal(out[r0:r1].view(torch.uint8), o.view(torch.uint8)), f'codes of rows {r0}..{r1}'
+        assert torch.equal(sf[r0:r1], s), f'scales of rows {r0}..{r1}'
+        og = tk.quant.per_token_cast_with_precomputed_sf(x[r0:r1], fmt, group, s)
+        og = og[0] if isinstance(og, tuple) else og
+        assert torch.equal(given[r0:r1].view(torch.uint8), og.view(torch.uint8)), f'codes for given scales of rows {r0}..{r1}'
